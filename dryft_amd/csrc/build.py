@@ -26,7 +26,7 @@ ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 MODULES = ("batch", "embed", "norm", "activation", "rope_kv", "attn_rows", "attn_mfma", "gemm", "sampling", "mlstm",
-           "rglru", "hyper", "wkv", "latent", "moe")
+           "rglru", "hyper", "wkv", "latent", "moe", "conv", "ssm", "delta")
 _HEADERS = ("common.h",)                       # every library includes these
 _OWN_HEADERS = {"sampling": ("sampling.h",)}    # and some a header of their own
 

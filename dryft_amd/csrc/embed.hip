@@ -16,6 +16,29 @@ __global__ void embed_rows_kernel(const int* __restrict__ tokens, const T* __res
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
 }
 
+// The same gather times a factor, as float32: the start of a float32 residual stream, out[r, :] = table[tokens[r], :] * scale.
+template <typename T>
+__global__ void embed_scaled_kernel(const int* __restrict__ tokens, const T* __restrict__ table, float* __restrict__ out,
+                                    int hidden, int vocab, float scale) {
+  int tok = tokens[blockIdx.x];
+  tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+  const T* src = table + (int64_t)tok * hidden;
+  float* dst = out + (int64_t)blockIdx.x * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = load_as_float(src + i) * scale;
+}
+
+DRYFT_API int dryft_embed_scaled(const int* tokens, const void* table, float* out, int n_rows, int hidden, int vocab,
+                                 float scale, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (is_f32)
+    hipLaunchKernelGGL(embed_scaled_kernel<float>, dim3(n_rows), dim3(256), 0, stream, tokens, (const float*)table, out,
+                       hidden, vocab, scale);
+  else
+    hipLaunchKernelGGL(embed_scaled_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, stream, tokens, (const bf16_t*)table, out,
+                       hidden, vocab, scale);
+  return DRYFT_LAUNCH_CHECK();
+}
+
 DRYFT_API int dryft_embed_rows(const int* tokens, const void* table, void* out, int n_rows, int hidden, int vocab,
                                int tables, int is_f32, hipStream_t stream) {
   if (n_rows <= 0 || tables <= 0) return 0;

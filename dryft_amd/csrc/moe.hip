@@ -176,11 +176,35 @@ DRYFT_API int dryft_moe_plan(const int* chosen, int n_pairs, int n_experts, int*
 }
 
 // ---------------------------------------------------------------------------------------------------
+// A router that is a table: row r's experts are the `top` entries of the table's row of its token id, each with
+// weight 1 / top.
+__global__ __launch_bounds__(256) void moe_table_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table,
+                                                              int* __restrict__ chosen, float* __restrict__ weights,
+                                                              int n_pairs, int top, int vocab, int n_experts) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_pairs) return;
+  const int tok = min(max(tokens[i / top], 0), vocab - 1);
+  chosen[i] = min(max(table[(int64_t)tok * top + i % top], 0), n_experts - 1);
+  weights[i] = 1.f / (float)top;
+}
+
+DRYFT_API int dryft_moe_table_route(const int* tokens, const int* table, int* chosen, float* weights, int rows, int top,
+                                    int vocab, int n_experts, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (top <= 0 || vocab <= 0 || n_experts <= 0) return -1;
+  const int n = rows * top;
+  hipLaunchKernelGGL(moe_table_route_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, tokens, table, chosen, weights,
+                     n, top, vocab, n_experts);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------
 // Grouped product, plain multiply-adds: for every tile of an expert's places, out[place] = W_e a[place]. A
 // workgroup takes one tile (up to 64 places) and 64 outputs; K goes through LDS 32 at a time; a thread owns four
 // places and four outputs. With `top` > 0 the operand rows are gathered: place -> pair -> row pair / top of `a`;
 // otherwise `a` is already in place order. GLU: W_e holds gate rows then up rows; the clamped gated unit
-// g * sigmoid(alpha g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit), is applied to the float
+// g * sigmoid(alpha g) * (u + offset), g = min(gate, limit), u = clamp(up, -limit, limit) (offset 0, alpha 1 and an
+// infinite limit make it silu(gate) * up), is applied to the float
 // accumulators and `n_out` counts its outputs.
 #define MOE_TN 64
 #define MOE_TK 32
@@ -192,7 +216,7 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
                                                           const int* __restrict__ tile_start,
                                                           const int* __restrict__ tile_rows,
                                                           const int* __restrict__ n_tiles, O* __restrict__ out, int top,
-                                                          int n_out, int k_dim, float limit, float alpha) {
+                                                          int n_out, int k_dim, float limit, float alpha, float offset) {
   __shared__ float sa[MOE_TILE][MOE_TK + 1];
   __shared__ float sw[(GLU ? 2 : 1) * MOE_TN][MOE_TK + 1];
   __shared__ int src_row[MOE_TILE];
@@ -255,7 +279,7 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
         // the unit reads what the products would have stored in the activation dtype
         const float g = fminf(rounded_as<T>(v), limit);
         const float u = fminf(fmaxf(rounded_as<T>(acc_up[i][j]), -limit), limit);
-        v = g / (1.f + expf(-alpha * g)) * (u + 1.f);
+        v = g / (1.f + expf(-alpha * g)) * (u + offset);
       }
       store_from_float(out + (int64_t)(start + r) * n_out + n, v);
     }
@@ -285,7 +309,7 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
                                                                const int* __restrict__ tile_start,
                                                                const int* __restrict__ tile_rows,
                                                                const int* __restrict__ n_tiles, O* __restrict__ out,
-                                                               int top, int n_out, int k_dim, float limit, float alpha) {
+                                                               int top, int n_out, int k_dim, float limit, float alpha, float offset) {
   constexpr int MT = MOE_TILE / 16;
   __shared__ __attribute__((aligned(16))) bf16_t sx[2][MOE_TILE * MOE_X_STRIDE];
   const int tile = blockIdx.x;
@@ -356,7 +380,7 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
       if (GLU) {
         const float gv = fminf(rounded_as<bf16_t>(v), limit);
         const float uv = fminf(fmaxf(rounded_as<bf16_t>(acc_up[mt][i]), -limit), limit);
-        v = gv / (1.f + expf(-alpha * gv)) * (uv + 1.f);
+        v = gv / (1.f + expf(-alpha * gv)) * (uv + offset);
       }
       store_from_float(out + (int64_t)(start + m) * n_out + n, v);
     }
@@ -375,7 +399,7 @@ __global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __re
                                                               const int* __restrict__ tile_start,
                                                               const int* __restrict__ tile_rows,
                                                               const int* __restrict__ n_tiles, O* __restrict__ out,
-                                                              int top, int n_out, int k_dim, float limit, float alpha) {
+                                                              int top, int n_out, int k_dim, float limit, float alpha, float offset) {
   const int tile = blockIdx.x;
   if (tile >= *n_tiles) return;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
@@ -421,7 +445,7 @@ __global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __re
       if (GLU) {
         const float gv = fminf(rounded_as<bf16_t>(v), limit);
         const float uv = fminf(fmaxf(rounded_as<bf16_t>(acc_up[i]), -limit), limit);
-        v = gv / (1.f + expf(-alpha * gv)) * (uv + 1.f);
+        v = gv / (1.f + expf(-alpha * gv)) * (uv + offset);
       }
       store_from_float(out + (int64_t)(start + m) * n_out + n, v);
     }
@@ -431,7 +455,7 @@ __global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __re
 DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, const int* sorted_pair,
                                 const int* tile_expert, const int* tile_start, const int* tile_rows, const int* n_tiles,
                                 int max_tiles, void* out, int out_is_f32, int top, int n_out, int k_dim, int glu,
-                                float limit, float alpha, int most_places, int is_f32, hipStream_t stream) {
+                                float limit, float alpha, float offset, int most_places, int is_f32, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || k_dim <= 0 || (glu && out_is_f32 && !is_f32)) return -1;
   dim3 grid(max_tiles, (n_out + MOE_TN - 1) / MOE_TN), block(256);
@@ -440,7 +464,7 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
 #define MOE_FEW(O, G)                                                                                             \
   hipLaunchKernelGGL((moe_product_few_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,           \
                      (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \
-                     k_dim, limit, alpha)
+                     k_dim, limit, alpha, offset)
       if (glu) MOE_FEW(bf16_t, true);
       else if (out_is_f32) MOE_FEW(float, false);
       else MOE_FEW(bf16_t, false);
@@ -450,7 +474,7 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
 #define MOE_MFMA(O, G)                                                                                            \
   hipLaunchKernelGGL((moe_product_mfma_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,          \
                      (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \
-                     k_dim, limit, alpha)
+                     k_dim, limit, alpha, offset)
     if (glu) MOE_MFMA(bf16_t, true);
     else if (out_is_f32) MOE_MFMA(float, false);
     else MOE_MFMA(bf16_t, false);
@@ -459,7 +483,7 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
   }
 #define MOE_LAUNCH(T, O, G)                                                                                       \
   hipLaunchKernelGGL((moe_product_kernel<T, O, G>), grid, block, 0, stream, (const T*)a, a_stride, (const T*)w,   \
-                     sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, k_dim, limit, alpha)
+                     sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, k_dim, limit, alpha, offset)
   if (is_f32) {
     if (glu) MOE_LAUNCH(float, float, true); else MOE_LAUNCH(float, float, false);
   } else if (glu) {
@@ -475,13 +499,14 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
 
 // ---------------------------------------------------------------------------------------------------
 // out[row] = sum_k weights[row, k] * y[place_of[row * top + k]]  (k in order)  + sigmoid(z_shared[row]) * shared[row]
+// (without logits the shared expert is added as it is)
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place_of,
                                                           const float* __restrict__ weights, const T* __restrict__ shared,
                                                           const float* __restrict__ logits, int64_t logit_stride,
                                                           int shared_col, T* __restrict__ out, int top, int width) {
   const int64_t row = blockIdx.x;
-  const float gate = shared ? 1.f / (1.f + expf(-logits[row * logit_stride + shared_col])) : 0.f;
+  const float gate = shared ? (logits ? 1.f / (1.f + expf(-logits[row * logit_stride + shared_col])) : 1.f) : 0.f;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     float acc = 0.f;
     for (int k = 0; k < top; ++k)

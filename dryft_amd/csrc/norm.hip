@@ -190,6 +190,9 @@ DRYFT_API int dryft_add_rows(const void* a, const void* b, void* out, int64_t n,
 // not at all, `extra` a row tensor in the activation dtype and `vec` one vector for every row. All of it
 // is float arithmetic; only y is rounded, once. The row is held in LDS between the passes (dynamic
 // shared memory of `width` floats), and a thread touches the same elements in every pass.
+// `form` chooses other norms: bit 0, the branch's norm takes the mean off first (a layer norm without bias:
+// (d - mean) * rsqrt(mean((d - mean)^2) + eps) * wb); bit 1, the same for y; bit 2, y is x_new itself, only rounded
+// (a sublayer that reads the stream as it is).
 template <typename T, typename D>
 __global__ __launch_bounds__(256) void stream_norm_kernel(const void* __restrict__ x_in, int x_kind,
                                                           const D* __restrict__ delta, int n_partials,
@@ -198,37 +201,56 @@ __global__ __launch_bounds__(256) void stream_norm_kernel(const void* __restrict
                                                           const void* __restrict__ vec, int vec_f32,
                                                           const void* __restrict__ w, int w_f32,
                                                           float* __restrict__ x_out, T* __restrict__ y, int width,
-                                                          float eps) {
+                                                          float eps, int form) {
   extern __shared__ __attribute__((aligned(16))) float held[];
   __shared__ float scratch[16];
   const int64_t base = (int64_t)blockIdx.x * width;
-  float inv_d = 1.f;
+  float inv_d = 1.f, mean_d = 0.f;
   if (n_partials > 0) {
-    float ss = 0.f;
+    float ss = 0.f, sd = 0.f;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
       float d = 0.f;
       for (int p = 0; p < n_partials; ++p) d += load_as_float(delta + p * partial_stride + base + i);
       held[i] = d;
       ss += d * d;
+      sd += d;
     }
-    if (wb != nullptr) inv_d = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+    if (wb != nullptr) {
+      if (form & 1) {
+        mean_d = block_sum(sd, scratch) / (float)width;
+        ss = 0.f;
+        for (int i = threadIdx.x; i < width; i += blockDim.x) { const float t = held[i] - mean_d; ss += t * t; }
+      }
+      inv_d = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+    }
   }
-  float ss = 0.f;
+  float ss = 0.f, sv = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float v = 0.f;
     if (x_kind == 2) v = ((const float*)x_in)[base + i];
     else if (x_kind == 1) v = load_as_float((const T*)x_in + base + i);
-    if (n_partials > 0) v += wb != nullptr ? held[i] * inv_d * load_vector(wb, i, wb_f32) : held[i];
+    if (n_partials > 0) v += wb != nullptr ? (held[i] - mean_d) * inv_d * load_vector(wb, i, wb_f32) : held[i];
     if (extra != nullptr) v += load_as_float(extra + base + i);
     if (vec != nullptr) v += load_vector(vec, i, vec_f32);
     held[i] = v;
     if (x_out != nullptr) x_out[base + i] = v;
     ss += v * v;
+    sv += v;
   }
   if (y == nullptr) return;
+  if (form & 4) {
+    for (int i = threadIdx.x; i < width; i += blockDim.x) store_from_float(y + base + i, held[i]);
+    return;
+  }
+  float mean = 0.f;
+  if (form & 2) {
+    mean = block_sum(sv, scratch) / (float)width;
+    ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) { const float t = held[i] - mean; ss += t * t; }
+  }
   const float inv = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
   for (int i = threadIdx.x; i < width; i += blockDim.x)
-    store_from_float(y + base + i, held[i] * inv * load_vector(w, i, w_f32));
+    store_from_float(y + base + i, (held[i] - mean) * inv * load_vector(w, i, w_f32));
 }
 
 // The same for rows whose width is a multiple of 8 with 16-byte aligned operands: a thread owns runs of 8
@@ -242,13 +264,13 @@ __global__ __launch_bounds__(256) void stream_norm_vec_kernel(const void* __rest
                                                               const void* __restrict__ vec, int vec_f32,
                                                               const void* __restrict__ w, int w_f32,
                                                               float* __restrict__ x_out, T* __restrict__ y, int width,
-                                                              float eps) {
+                                                              float eps, int form) {
   extern __shared__ __attribute__((aligned(16))) float held[];
   __shared__ float scratch[16];
   const int64_t base = (int64_t)blockIdx.x * width;
-  float inv_d = 1.f;
+  float inv_d = 1.f, mean_d = 0.f;
   if (n_partials > 0) {
-    float ss = 0.f;
+    float ss = 0.f, sd = 0.f;
     for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
       float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       int p = 0;
@@ -268,12 +290,24 @@ __global__ __launch_bounds__(256) void stream_norm_vec_kernel(const void* __rest
         for (int j = 0; j < 8; ++j) d[j] += t[j];
       }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) ss += d[j] * d[j];
+      for (int j = 0; j < 8; ++j) { ss += d[j] * d[j]; sd += d[j]; }
       store8_from_float(held + i, d);
     }
-    if (wb != nullptr) inv_d = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+    if (wb != nullptr) {
+      if (form & 1) {
+        mean_d = block_sum(sd, scratch) / (float)width;
+        ss = 0.f;
+        for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+          float d[8];
+          load8_as_float(held + i, d);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ss += (d[j] - mean_d) * (d[j] - mean_d);
+        }
+      }
+      inv_d = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
+    }
   }
-  float ss = 0.f;
+  float ss = 0.f, sv = 0.f;
   for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
     float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, t[8];
     if (x_kind == 2) load8_as_float((const float*)x_in + base + i, v);
@@ -284,7 +318,7 @@ __global__ __launch_bounds__(256) void stream_norm_vec_kernel(const void* __rest
         float wv[8];
         if (wb_f32) load8_as_float((const float*)wb + i, wv); else load8_as_float((const bf16_t*)wb + i, wv);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] += t[j] * inv_d * wv[j];
+        for (int j = 0; j < 8; ++j) v[j] += (t[j] - mean_d) * inv_d * wv[j];
       } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] += t[j];
@@ -303,16 +337,35 @@ __global__ __launch_bounds__(256) void stream_norm_vec_kernel(const void* __rest
     store8_from_float(held + i, v);
     if (x_out != nullptr) store8_from_float(x_out + base + i, v);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+    for (int j = 0; j < 8; ++j) { ss += v[j] * v[j]; sv += v[j]; }
   }
   if (y == nullptr) return;
+  if (form & 4) {
+    for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+      float v[8];
+      load8_as_float(held + i, v);
+      store8_from_float(y + base + i, v);
+    }
+    return;
+  }
+  float mean = 0.f;
+  if (form & 2) {
+    mean = block_sum(sv, scratch) / (float)width;
+    ss = 0.f;
+    for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+      float v[8];
+      load8_as_float(held + i, v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += (v[j] - mean) * (v[j] - mean);
+    }
+  }
   const float inv = rsqrtf(block_sum(ss, scratch) / (float)width + eps);
   for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
     float v[8], wv[8];
     load8_as_float(held + i, v);
     if (w_f32) load8_as_float((const float*)w + i, wv); else load8_as_float((const bf16_t*)w + i, wv);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] *= inv * wv[j];
+    for (int j = 0; j < 8; ++j) v[j] = (v[j] - mean) * inv * wv[j];
     store8_from_float(y + base + i, v);
   }
 }
@@ -324,20 +377,20 @@ __global__ __launch_bounds__(256) void stream_norm_vec_kernel(const void* __rest
 DRYFT_API int dryft_stream_norm(const void* x_in, int x_kind, const void* delta, int delta_kind, int n_partials,
                                 int64_t partial_stride, const void* wb, int wb_f32, const void* extra,
                                 const void* vec, int vec_f32, const void* w, int w_f32, float* x_out, void* y,
-                                int n_rows, int width, float eps, int is_f32, hipStream_t stream) {
+                                int n_rows, int width, float eps, int is_f32, int form, hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (width <= 0 || width > STREAM_NORM_MAX_WIDTH || (y != nullptr && w == nullptr)) return -1;
+  if (width <= 0 || width > STREAM_NORM_MAX_WIDTH || (y != nullptr && w == nullptr && !(form & 4))) return -1;
   if (delta_kind == 0) n_partials = 0;
   dim3 grid(n_rows), block(256);
   const size_t lds = (size_t)width * sizeof(float);
 #define SN(TT, DD)                                                                                                   \
   hipLaunchKernelGGL((stream_norm_kernel<TT, DD>), grid, block, lds, stream, x_in, x_kind, (const DD*)delta,        \
                      n_partials, partial_stride, wb, wb_f32, (const TT*)extra, vec, vec_f32, w, w_f32, x_out,       \
-                     (TT*)y, width, eps)
+                     (TT*)y, width, eps, form)
 #define SNV(TT, DD)                                                                                                  \
   hipLaunchKernelGGL((stream_norm_vec_kernel<TT, DD>), grid, block, lds, stream, x_in, x_kind, (const DD*)delta,    \
                      n_partials, partial_stride, wb, wb_f32, (const TT*)extra, vec, vec_f32, w, w_f32, x_out,       \
-                     (TT*)y, width, eps)
+                     (TT*)y, width, eps, form)
   const bool aligned = (((uintptr_t)x_in | (uintptr_t)delta | (uintptr_t)wb | (uintptr_t)extra | (uintptr_t)vec |
                          (uintptr_t)w | (uintptr_t)x_out | (uintptr_t)y) & 15) == 0 && partial_stride % 4 == 0;
   if (width % 8 == 0 && aligned) {
@@ -351,5 +404,59 @@ DRYFT_API int dryft_stream_norm(const void* x_in, int x_kind, const void* delta,
   else if (delta_kind == 2) SN(bf16_t, float);
   else SN(bf16_t, bf16_t);
 #undef SN
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The mean of two branches that are each normed first: per row
+//
+//   a = sum_p A[p] (+ bias_a),  b = sum_p B[p] (+ bias_b)        (a branch's output: T, or float partial sums)
+//   out = ( a * rsqrt(mean(a^2) + eps) * wa  +  b * rsqrt(mean(b^2) + eps) * wb ) / 2
+//
+// in float, stored as float32 (the consumer norms it once more before it enters the stream). Both rows wait in LDS
+// (dynamic shared memory of 2 * width floats).
+template <typename DA, typename DB>
+__global__ __launch_bounds__(256) void rms_pair_mean_kernel(const DA* __restrict__ a, int a_parts, int64_t a_stride,
+                                                            const float* __restrict__ a_bias, const float* __restrict__ wa,
+                                                            const DB* __restrict__ b, int b_parts, int64_t b_stride,
+                                                            const float* __restrict__ b_bias, const float* __restrict__ wb,
+                                                            float* __restrict__ out, int width, float eps) {
+  extern __shared__ __attribute__((aligned(16))) float held[];
+  __shared__ float scratch[16];
+  const int64_t base = (int64_t)blockIdx.x * width;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float x = a_bias ? a_bias[i] : 0.f, y = b_bias ? b_bias[i] : 0.f;
+    for (int p = 0; p < a_parts; ++p) x += load_as_float(a + p * a_stride + base + i);
+    for (int p = 0; p < b_parts; ++p) y += load_as_float(b + p * b_stride + base + i);
+    held[i] = x;
+    held[width + i] = y;
+    sa += x * x;
+    sb += y * y;
+  }
+  const float inv_a = rsqrtf(block_sum(sa, scratch) / (float)width + eps);
+  const float inv_b = rsqrtf(block_sum(sb, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    out[base + i] = 0.5f * (held[i] * inv_a * wa[i] + held[width + i] * inv_b * wb[i]);
+}
+
+// a_kind / b_kind: 1 = activation dtype [rows, width], 2 = float partial sums [parts, rows, width].
+DRYFT_API int dryft_rms_pair_mean(const void* a, int a_kind, int a_parts, int64_t a_stride, const float* a_bias,
+                                  const float* wa, const void* b, int b_kind, int b_parts, int64_t b_stride,
+                                  const float* b_bias, const float* wb, float* out, int n_rows, int width, float eps,
+                                  int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (width <= 0 || 2 * width > STREAM_NORM_MAX_WIDTH || a_parts < 1 || b_parts < 1) return -1;
+  dim3 grid(n_rows), block(256);
+  const size_t lds = (size_t)2 * width * sizeof(float);
+  const bool fa = is_f32 || a_kind == 2, fb = is_f32 || b_kind == 2;
+#define PM(DA, DB)                                                                                                    \
+  hipLaunchKernelGGL((rms_pair_mean_kernel<DA, DB>), grid, block, lds, stream, (const DA*)a, a_parts, a_stride, a_bias, \
+                     wa, (const DB*)b, b_parts, b_stride, b_bias, wb, out, width, eps)
+  if (fa && fb) PM(float, float);
+  else if (fa) PM(float, bf16_t);
+  else if (fb) PM(bf16_t, float);
+  else PM(bf16_t, bf16_t);
+#undef PM
   return DRYFT_LAUNCH_CHECK();
 }

@@ -20,10 +20,12 @@ _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
     "batch": {"dryft_prepare_batch": [_P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _P],
               "dryft_tile_prefix": [_P, _P, _I, _I, _P, _P]},
-    "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _I, _P]},
+    "embed": {"dryft_embed_rows": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+              "dryft_embed_scaled": [_P, _P, _P, _I, _I, _I, _F, _I, _P]},
     "norm": {"dryft_add_rmsnorm": [_P, _P, _I, _I, _L, _P, _I, _P, _P, _I, _I, _F, _I, _P],
              "dryft_add_rows": [_P, _P, _P, _L, _I, _P],
-             "dryft_stream_norm": [_P, _I, _P, _I, _I, _L, _P, _I, _P, _P, _I, _P, _I, _P, _P, _I, _I, _F, _I, _P]},
+             "dryft_stream_norm": [_P, _I, _P, _I, _I, _L, _P, _I, _P, _P, _I, _P, _I, _P, _P, _I, _I, _F, _I, _I, _P],
+             "dryft_rms_pair_mean": [_P, _I, _I, _L, _P, _P, _P, _I, _I, _L, _P, _P, _P, _I, _I, _F, _I, _P]},
     "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P],
                    "dryft_glu_clamped": [_P, _P, _I, _I, _L, _F, _F, _I, _P],
                    "dryft_sigmoid_gate": [_P, _L, _P, _L, _P, _I, _I, _I, _P]},
@@ -43,6 +45,8 @@ _SIGNATURES = {
                                           _I, _I, _I, _I, _I, _P],
                 "dryft_rope_pairs_kv": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                         _I, _I, _P],
+                "dryft_norm_rope_half_kv": [_P, _L, _I, _I, _I, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I,
+                                            _I, _I, _I, _I, _I, _P],
                 "dryft_rows_to_cache_takes": [_I, _I, _I, _I],
                 "dryft_rows_to_cache_parts": [_P, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                               _I, _I, _I, _P]},
@@ -77,15 +81,25 @@ _SIGNATURES = {
             "dryft_wkv_decay": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
             "dryft_wkv_steps": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P, _I, _I, _P, _P, _I,
                                 _P],
-            "dryft_wkv_out": [_P, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
+            "dryft_wkv_out": [_P, _P, _P, _P, _I, _I, _I, _F, _L, _I, _P]},
     "latent": {"dryft_rms_segments": [_P, _L, _I, _P, _P, _I, _P, _P, _I, _F, _I, _I, _P],
                "dryft_latent_rope_kv": [_P, _P, _P, _L, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                         _I, _I, _I, _P],
                "dryft_head_gate": [_P, _P, _L, _I, _P, _I, _I, _I, _I, _I, _P]},
     "moe": {"dryft_moe_route": [_P, _L, _P, _I, _I, _I, _I, _F, _P, _P, _I, _P],
             "dryft_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
-            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
+            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _F, _I, _I, _P],
+            "dryft_moe_table_route": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
             "dryft_moe_combine": [_P, _P, _P, _P, _P, _L, _I, _P, _I, _I, _I, _I, _P]},
+    "conv": {"dryft_conv_max_taps": [],
+             "dryft_causal_conv": [_P, _L, _I, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+             "dryft_conv_tail": [_P, _L, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P]},
+    "ssm": {"dryft_ssm_max_state": [],
+            "dryft_ssm_scan": [_P, _L, _I, _I, _I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+            "dryft_gate_part_norm": [_P, _P, _L, _I, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
+    "delta": {"dryft_delta_max_dim": [],
+              "dryft_delta_steps": [_P, _L, _I, _I, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
+                                    _F, _F, _I, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
                  "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _I, _P, _P, _P]},
 }
@@ -245,8 +259,11 @@ def add_rows(a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tenso
     return out
 
 
-def stream_norm(x, delta, post_weight, extra, vec, weight, eps: float, x_out, y, act: torch.dtype) -> None:
-    """The norms of a float32 residual stream in one launch, per row:
+def stream_norm(x, delta, post_weight, extra, vec, weight, eps: float, x_out, y, act: torch.dtype,
+                post_centred: bool = False, centred: bool = False, plain_read: bool = False) -> None:
+    """The norms of a float32 residual stream in one launch, per row (``post_centred`` / ``centred``: the norm of
+    ``d`` / of ``x_out`` takes the mean off first and divides by the standard deviation, a layer norm without bias;
+    ``plain_read``: ``y`` is ``x_out`` itself in the activation dtype, no weight):
     ``d = delta`` (a tensor in the activation dtype, or ``[n, rows, width]`` float32 partial sums as ``(data, n)``);
     ``x_out = x + rmsnorm(d) * post_weight + extra + vec`` (each term optional; without ``post_weight`` ``d`` is added
     as it is); ``y = rmsnorm(x_out) * weight`` in the activation dtype (optional). ``x`` is float32, or in the
@@ -292,13 +309,13 @@ def stream_norm(x, delta, post_weight, extra, vec, weight, eps: float, x_out, y,
             raise KernelError("stream_norm: x_out must be contiguous float32 [rows, width]")
     if y is not None:
         _gpu(y, "y", act)
-        if not (y.is_contiguous() and weight is not None):
+        if not (y.is_contiguous() and (weight is not None or plain_read)):
             raise KernelError("stream_norm: y contiguous, and a weight for it")
     flag = lambda t: 0 if t is None else _float_flag(t, "vector")      # noqa: E731
     _check(_fn("norm", "dryft_stream_norm")(
         _ptr(x), x_kind, _ptr(delta), kind, n_partials, stride, _ptr(post_weight), flag(post_weight), _ptr(extra),
         _ptr(vec), flag(vec), _ptr(weight), flag(weight), _ptr(x_out), _ptr(y), rows, width, float(eps), is_f32,
-        _stream()), "stream_norm")
+        (1 if post_centred else 0) | (2 if centred else 0) | (4 if plain_read else 0), _stream()), "stream_norm")
 
 
 # -------------------------------------------------------------------------------------- activation
@@ -1463,18 +1480,21 @@ def wkv_steps(r, k, v, decay, bonus, seq_slot, cu_rows, q_len, n_seqs: int, stat
 
 
 def wkv_out(o_raw, gate, weight, out, n_heads: int, dim: int, eps: float) -> None:
-    """``out = o_raw / rms_per_head(o_raw) * weight * silu(gate)`` in the activation dtype."""
+    """``out = o_raw / rms_per_head(o_raw) * weight * silu(gate)`` in the activation dtype; ``gate`` may be a run of
+    columns of a wider tensor."""
     _gpu(gate, "gate")
     rows = gate.shape[0]
     inner = n_heads * dim
     _gpu(o_raw, "o_raw", torch.float32)
     _gpu(out, "out", gate.dtype)
-    for name, t in (("o_raw", o_raw), ("gate", gate), ("out", out)):
+    for name, t in (("o_raw", o_raw), ("out", out)):
         if not (t.shape == (rows, inner) and t.is_contiguous()):
             raise KernelError(f"wkv_out: {name} must be contiguous [rows, {inner}]")
+    if not (gate.shape == (rows, inner) and gate.stride(1) == 1):
+        raise KernelError(f"wkv_out: gate must be [rows, {inner}] with unit column stride")
     _f32_vector(weight, "weight", inner)
     _check(_fn("wkv", "dryft_wkv_out")(_ptr(o_raw), _ptr(gate), _ptr(weight), _ptr(out), rows, n_heads, dim, float(eps),
-                                       _float_flag(gate, "gate"), _stream()), "wkv_out")
+                                       gate.stride(0), _float_flag(gate, "gate"), _stream()), "wkv_out")
 
 
 # ------------------------------------------------------------------------------------------ latent attention
@@ -1609,11 +1629,28 @@ def moe_plan(chosen, n_experts: int) -> MoePlan:
     return plan
 
 
-def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple[float, float] | None = None) -> None:
+def moe_table_route(tokens, table, n_experts: int, chosen, weights) -> None:
+    """A router that is a table: row ``r`` goes to the experts ``table[tokens[r]]`` (int32 ``[vocab, top]``), each with
+    weight ``1 / top``. ``chosen`` int32 and ``weights`` float32 ``[rows, top]``."""
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(table, "table", torch.int32)
+    _gpu(chosen, "chosen", torch.int32)
+    _gpu(weights, "weights", torch.float32)
+    rows, top = chosen.shape
+    if not (tokens.is_contiguous() and tokens.numel() == rows and table.dim() == 2 and table.shape[1] == top and
+            table.is_contiguous() and chosen.is_contiguous() and weights.shape == (rows, top) and weights.is_contiguous()):
+        raise KernelError("moe_table_route: tokens [rows], table [vocab, top], chosen and weights [rows, top], contiguous")
+    _check(_fn("moe", "dryft_moe_table_route")(_ptr(tokens), _ptr(table), _ptr(chosen), _ptr(weights), rows, top,
+                                               table.shape[0], n_experts, _stream()), "moe_table_route")
+
+
+def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple | None = None) -> None:
     """``out[place] = W_e a_row`` for every place of the plan, ``e`` the place's expert. ``top`` > 0: ``a`` is
     ``[rows, K]`` and a place's operand is row ``pair // top``; ``top`` == 0: ``a`` is ``[pairs, K]`` in place order.
     ``w`` is ``[experts, N, K]``; with ``glu = (limit, alpha)`` it holds gate rows then up rows (``N = 2 I``) and
-    ``out [pairs, I]`` receives the clamped gated unit of the two. ``out`` may be float32 for a plain product."""
+    ``out [pairs, I]`` receives the clamped gated unit of the two, ``g sigmoid(alpha g) (u + 1)``; ``glu = (limit, alpha,
+    offset)`` puts ``offset`` in the place of that 1 (``(inf, 1, 0)`` is ``silu(gate) * up``). ``out`` may be float32
+    for a plain product."""
     _gpu(a, "a")
     _gpu(w, "w", a.dtype)
     _gpu(out, "out")
@@ -1629,17 +1666,18 @@ def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple[float, float] | 
         raise KernelError(f"moe_products: out must be contiguous [{plan.n_pairs}, {n_out}] in a's dtype or float32")
     if glu and out.dtype != a.dtype:
         raise KernelError("moe_products: the gated unit is stored in the activation dtype")
-    limit, alpha = glu if glu else (0.0, 0.0)
+    limit, alpha, offset = (tuple(glu) + (1.0,))[:3] if glu else (0.0, 0.0, 0.0)
     _check(_fn("moe", "dryft_moe_product")(
         _ptr(a), a.stride(0), _ptr(w), _ptr(plan.sorted_pair), _ptr(plan.tiles[0]), _ptr(plan.tiles[1]),
         _ptr(plan.tiles[2]), _ptr(plan.n_tiles), plan.max_tiles, _ptr(out), 1 if out.dtype == torch.float32 else 0,
-        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), plan.most_places, _float_flag(a, "a"), _stream()),
+        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), float(offset), plan.most_places,
+        _float_flag(a, "a"), _stream()),
         "moe_products")
 
 
 def moe_combine(y, plan: MoePlan, weights, shared, logits, shared_col: int, out) -> None:
     """``out[row] = sum_k weights[row, k] * y[place of (row, k)] + sigmoid(logits[row, shared_col]) * shared[row]``
-    (the last term only with ``shared``)."""
+    (the last term only with ``shared``; without ``logits`` the shared expert's output is added as it is)."""
     _gpu(y, "y", torch.float32)
     rows, top = weights.shape
     width = y.shape[1]
@@ -1650,10 +1688,260 @@ def moe_combine(y, plan: MoePlan, weights, shared, logits, shared_col: int, out)
         raise KernelError("moe_combine: y [pairs, width], weights [rows, top], out [rows, width], all contiguous")
     if shared is not None:
         _gpu(shared, "shared", out.dtype)
+        if not (shared.shape == (rows, width) and shared.is_contiguous()):
+            raise KernelError("moe_combine: shared [rows, width] contiguous")
+    if shared is not None and logits is not None:
         _gpu(logits, "logits", torch.float32)
-        if not (shared.shape == (rows, width) and shared.is_contiguous() and logits.stride(1) == 1 and
-                0 <= shared_col < logits.shape[1] and logits.shape[0] == rows):
-            raise KernelError("moe_combine: shared [rows, width] contiguous, its logit a column of logits")
+        if not (logits.stride(1) == 1 and 0 <= shared_col < logits.shape[1] and logits.shape[0] == rows):
+            raise KernelError("moe_combine: the shared expert's logit must be a column of logits")
     _check(_fn("moe", "dryft_moe_combine")(_ptr(y), _ptr(plan.place_of), _ptr(weights), _ptr(shared), _ptr(logits),
-                                           logits.stride(0) if shared is not None else 0, shared_col, _ptr(out), rows, top,
+                                           logits.stride(0) if (shared is not None and logits is not None) else 0, shared_col, _ptr(out), rows, top,
                                            width, _float_flag(out, "out"), _stream()), "moe_combine")
+
+
+# ------------------------------------------------------------------------------- scaled embedding, pair of branches
+def embed_scaled(tokens: torch.Tensor, table: torch.Tensor, scale: float, out: torch.Tensor) -> torch.Tensor:
+    """``out[r] = table[tokens[r]] * scale`` as float32: the start of a float32 residual stream."""
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(table, "table")
+    _gpu(out, "out", torch.float32)
+    n = tokens.numel()
+    if not (table.dim() == 2 and table.is_contiguous() and tokens.is_contiguous() and out.is_contiguous() and
+            out.shape == (n, table.shape[1])):
+        raise KernelError("embed_scaled: table [vocab, hidden], out float32 [rows, hidden], all contiguous")
+    _check(_fn("embed", "dryft_embed_scaled")(_ptr(tokens), _ptr(table), _ptr(out), n, table.shape[1], table.shape[0],
+                                              float(scale), _float_flag(table, "table"), _stream()), "embed_scaled")
+    return out
+
+
+def _branch(delta, rows: int, width: int, act: torch.dtype, what: str):
+    """(pointer, kind, parts, stride) of a branch's output: a tensor ``[rows, width]`` in the activation dtype, or float32
+    partial sums ``(data [n, rows, width], n)``."""
+    if isinstance(delta, tuple):
+        data, n = delta
+        _gpu(data, what, torch.float32)
+        if not (data.dim() == 3 and data.shape[1:] == (rows, width) and data.is_contiguous() and data.shape[0] >= n >= 1):
+            raise KernelError(f"{what}: partial sums must be contiguous float32 [n, rows, width]")
+        return data, 2, int(n), rows * width
+    _gpu(delta, what, act)
+    if not (delta.shape == (rows, width) and delta.is_contiguous()):
+        raise KernelError(f"{what}: must be contiguous [rows, width] in the activation dtype")
+    return delta, 1, 1, rows * width
+
+
+def rms_pair_mean(a, a_bias, a_weight, b, b_bias, b_weight, eps: float, out: torch.Tensor, act: torch.dtype) -> torch.Tensor:
+    """``out = (rmsnorm(a + a_bias) * a_weight + rmsnorm(b + b_bias) * b_weight) / 2`` per row, float32. ``a`` and ``b``
+    are tensors in the activation dtype ``act`` or float32 partial sums ``(data, n)``; biases (optional) and weights
+    are float32 vectors."""
+    _gpu(out, "out", torch.float32)
+    rows, width = out.shape
+    if not out.is_contiguous():
+        raise KernelError("rms_pair_mean: out must be contiguous")
+    pa, ka, na, sa = _branch(a, rows, width, act, "a")
+    pb, kb, nb, sb = _branch(b, rows, width, act, "b")
+    for name, t in (("a_bias", a_bias), ("b_bias", b_bias)):
+        if t is not None:
+            _f32_vector(t, name, width)
+    _f32_vector(a_weight, "a_weight", width)
+    _f32_vector(b_weight, "b_weight", width)
+    _check(_fn("norm", "dryft_rms_pair_mean")(_ptr(pa), ka, na, sa, _ptr(a_bias), _ptr(a_weight), _ptr(pb), kb, nb, sb,
+                                              _ptr(b_bias), _ptr(b_weight), _ptr(out), rows, width, float(eps),
+                                              1 if act == torch.float32 else 0, _stream()), "rms_pair_mean")
+    return out
+
+
+# --------------------------------------------------------------------------------------- short causal convolution
+CONV_MAX_TAPS = 16
+
+
+def _row_facts(rows: int, **tensors) -> None:
+    for name, t in tensors.items():
+        _gpu(t, name, torch.int32)
+        if not (t.is_contiguous() and t.numel() >= rows):
+            raise KernelError(f"{name}: needs {rows} contiguous entries")
+
+
+def causal_conv(u, col: int, channels: int, in_bias, weight, out_bias, silu: bool, row_slot, row_seq, row_pos, seq_start,
+                tail, out) -> torch.Tensor:
+    """``out[t, c] = act(sum_j weight[c, j] * v[t - taps + 1 + j, c] + out_bias[c])`` with ``v = u[:, col + c] + in_bias[c]``
+    over each sequence's own rows, the ``taps - 1`` inputs before the step's first row from ``tail [slots, taps - 1,
+    channels]`` (float32), zeros before the sequence's start. ``act`` is the identity or (``silu``) ``z sigmoid(z)``.
+    Rows of sequences that sit out give zeros. The tail is not touched (``conv_tail`` moves it on)."""
+    _gpu(u, "u")
+    rows = u.shape[0]
+    if not (u.dim() == 2 and u.stride(1) == 1 and 0 <= col and col + channels <= u.shape[1]):
+        raise KernelError("causal_conv: u [rows, columns] with unit column stride that holds the channels")
+    _gpu(weight, "weight", torch.float32)
+    if not (weight.dim() == 2 and weight.shape[0] == channels and weight.is_contiguous() and
+            1 <= weight.shape[1] <= CONV_MAX_TAPS):
+        raise KernelError(f"causal_conv: weight must be contiguous float32 [channels, 1..{CONV_MAX_TAPS}]")
+    taps = weight.shape[1]
+    for name, t in (("in_bias", in_bias), ("out_bias", out_bias)):
+        if t is not None:
+            _f32_vector(t, name, channels)
+    _row_facts(rows, row_slot=row_slot, row_seq=row_seq, row_pos=row_pos)
+    _gpu(seq_start, "seq_start", torch.int32)
+    if taps > 1:
+        _gpu(tail, "tail", torch.float32)
+        if not (tail.dim() == 3 and tail.shape[1:] == (taps - 1, channels) and tail.is_contiguous()):
+            raise KernelError(f"causal_conv: tail must be contiguous float32 [slots, {taps - 1}, {channels}]")
+    _gpu(out, "out", u.dtype)
+    if not (out.shape == (rows, channels) and out.is_contiguous()):
+        raise KernelError("causal_conv: out must be contiguous [rows, channels]")
+    _check(_fn("conv", "dryft_causal_conv")(_ptr(u), u.stride(0), col, _ptr(in_bias), _ptr(weight), _ptr(out_bias), taps,
+                                            1 if silu else 0, _ptr(row_slot), _ptr(row_seq), _ptr(row_pos),
+                                            _ptr(seq_start), _ptr(tail) if taps > 1 else 0, _ptr(out), rows, channels,
+                                            _float_flag(u, "u"), _stream()), "causal_conv")
+    return out
+
+
+def conv_tail(u, col: int, channels: int, in_bias, taps: int, seq_slot, cu_rows, q_len, n_seqs: int, tail) -> None:
+    """Moves each sequence's tail on past the step's rows: afterwards it holds the last ``taps - 1`` inputs
+    ``u[:, col + c] + in_bias[c]`` of the sequence (older ones from the tail before where the step brought fewer)."""
+    if taps <= 1:
+        return
+    _gpu(u, "u")
+    if not (u.dim() == 2 and u.stride(1) == 1 and 0 <= col and col + channels <= u.shape[1]):
+        raise KernelError("conv_tail: u [rows, columns] with unit column stride that holds the channels")
+    if in_bias is not None:
+        _f32_vector(in_bias, "in_bias", channels)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    _gpu(tail, "tail", torch.float32)
+    if not (tail.dim() == 3 and tail.shape[1:] == (taps - 1, channels) and tail.is_contiguous() and taps <= CONV_MAX_TAPS):
+        raise KernelError(f"conv_tail: tail must be contiguous float32 [slots, {taps - 1}, {channels}]")
+    _check(_fn("conv", "dryft_conv_tail")(_ptr(u), u.stride(0), col, _ptr(in_bias), taps, _ptr(seq_slot), _ptr(cu_rows),
+                                          _ptr(q_len), _ptr(tail), n_seqs, channels, _float_flag(u, "u"), _stream()),
+           "conv_tail")
+
+
+# ------------------------------------------------------------------------- norm per head, rotation over halves, append
+def norm_rope_half_kv(src, q_col: int, k_col: int, v_col: int, q_weight, k_weight, eps: float, cos, sin, rot: int,
+                      row_slot, row_pos, q_out, k_pages, v_pages, page_table, write_kv: bool, n_heads: int, n_kv: int,
+                      head_dim: int, v_dim: int) -> None:
+    """Every q and k head of ``src`` divided by its root mean square and multiplied by ``q_weight`` / ``k_weight``
+    (float32 ``[head_dim]``; None: the head passes), then feature ``i`` of its first ``rot`` turned with feature
+    ``i + rot / 2`` by float32 tables ``[positions, rot / 2]``; queries to ``q_out [rows, heads, head_dim]`` and, when
+    ``write_kv``, keys and (untouched) values of width ``v_dim`` to their pages."""
+    _gpu(src, "src")
+    is_f32 = _float_flag(src, "src")
+    rows = src.shape[0]
+    if not (src.dim() == 2 and src.stride(1) == 1):
+        raise KernelError("norm_rope_half_kv: src must be [rows, columns] with unit column stride")
+    ends = (q_col + n_heads * head_dim, k_col + n_kv * head_dim, v_col + n_kv * v_dim)
+    if min(q_col, k_col, v_col) < 0 or max(ends) > src.shape[1]:
+        raise KernelError("norm_rope_half_kv: q, k or v lie outside the columns of src")
+    if rot % 2 or not 0 <= rot <= head_dim or head_dim > 256:
+        raise KernelError(f"norm_rope_half_kv: the rotated width must be even and at most {head_dim} <= 256, got {rot}")
+    if rot:
+        for name, t in (("cos", cos), ("sin", sin)):
+            _gpu(t, name, torch.float32)
+            if not (t.dim() == 2 and t.shape[1] == rot // 2 and t.is_contiguous()):
+                raise KernelError(f"{name}: must be contiguous float32 [positions, {rot // 2}]")
+    for name, t in (("q_weight", q_weight), ("k_weight", k_weight)):
+        if t is not None:
+            _f32_vector(t, name, head_dim)
+    _gpu(q_out, "q_out", src.dtype)
+    if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim):
+        raise KernelError("norm_rope_half_kv: q_out must be [rows, heads, head_dim]")
+    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, src.dtype, v_dim)
+    _row_facts(rows, row_slot=row_slot, row_pos=row_pos)
+    _check(_fn("rope_kv", "dryft_norm_rope_half_kv")(
+        _ptr(src), src.stride(0), q_col, k_col, v_col, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos), _ptr(sin),
+        rot, _ptr(row_slot), _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
+        page_table.shape[1], int(bool(write_kv)), rows, n_heads, n_kv, head_dim, v_dim, is_f32, _stream()),
+        "norm_rope_half_kv")
+
+
+# ------------------------------------------------------------------------------------------ state-space mixer
+SSM_MAX_STATE = 256
+
+
+def ssm_scan(xbc, x_col: int, b_col: int, c_col: int, dt_raw, dt_bias, a_log, d_skip, seq_slot, cu_rows, q_len,
+             n_seqs: int, state, y, n_heads: int, head_dim: int, n_state: int, groups: int, write_state: bool) -> None:
+    """Per sequence and head, over the sequence's rows of the step in order, from ``state [slots, heads, n_state,
+    head_dim]`` (float32): ``dt = softplus(dt_raw + dt_bias)``, ``S <- exp(-exp(a_log) dt) S + dt B x^T``,
+    ``y = S^T C + d_skip x``. ``x [heads, head_dim]``, ``B`` and ``C [groups, n_state]`` are runs of columns of ``xbc``
+    (activation dtype), ``dt_raw`` float32 ``[rows, >= heads]``, ``y`` float32 ``[rows, heads * head_dim]`` (rows of
+    sequences that sit out are not written)."""
+    _gpu(xbc, "xbc")
+    rows = xbc.shape[0]
+    inner = n_heads * head_dim
+    if not (xbc.dim() == 2 and xbc.stride(1) == 1 and min(x_col, b_col, c_col) >= 0 and
+            max(x_col + inner, b_col + groups * n_state, c_col + groups * n_state) <= xbc.shape[1]):
+        raise KernelError("ssm_scan: x, B or C lie outside the columns of xbc")
+    _gpu(dt_raw, "dt_raw", torch.float32)
+    if not (dt_raw.dim() == 2 and dt_raw.shape[0] == rows and dt_raw.stride(1) == 1 and dt_raw.shape[1] >= n_heads):
+        raise KernelError("ssm_scan: dt_raw must be float32 [rows, >= heads] with unit column stride")
+    for name, t in (("dt_bias", dt_bias), ("a_log", a_log), ("d_skip", d_skip)):
+        _f32_vector(t, name, n_heads)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    _gpu(state, "state", torch.float32)
+    if not (state.dim() == 4 and state.shape[1:] == (n_heads, n_state, head_dim) and state.is_contiguous()):
+        raise KernelError(f"ssm_scan: state must be contiguous float32 [slots, {n_heads}, {n_state}, {head_dim}]")
+    _gpu(y, "y", torch.float32)
+    if not (y.shape == (rows, inner) and y.is_contiguous()):
+        raise KernelError("ssm_scan: y must be contiguous float32 [rows, heads * head_dim]")
+    if not (0 < n_state <= SSM_MAX_STATE and groups > 0 and n_heads % groups == 0):
+        raise KernelError(f"ssm_scan: a state of 1..{SSM_MAX_STATE} rows, heads a multiple of groups")
+    _check(_fn("ssm", "dryft_ssm_scan")(_ptr(xbc), xbc.stride(0), x_col, b_col, c_col, _ptr(dt_raw), dt_raw.stride(0),
+                                        _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(seq_slot), _ptr(cu_rows),
+                                        _ptr(q_len), _ptr(state), _ptr(y), n_seqs, n_heads, head_dim, n_state, groups,
+                                        int(bool(write_state)), _float_flag(xbc, "xbc"), _stream()), "ssm_scan")
+
+
+def gate_part_norm(y, z, z_col: int, weight, row_slot, out, parts: int, eps: float) -> None:
+    """``v = y * silu(z[:, z_col : z_col + inner])``, each of ``parts`` equal runs of ``v`` divided by its own root mean
+    square, times ``weight``: the gate comes before the norm. ``y`` float32, ``z`` and ``out`` in the activation dtype."""
+    _gpu(y, "y", torch.float32)
+    rows, inner = y.shape
+    _gpu(z, "z")
+    _gpu(out, "out", z.dtype)
+    if not (y.is_contiguous() and z.dim() == 2 and z.shape[0] == rows and z.stride(1) == 1 and 0 <= z_col and
+            z_col + inner <= z.shape[1] and out.shape == (rows, inner) and out.is_contiguous()):
+        raise KernelError("gate_part_norm: y and out contiguous [rows, inner], the gate a run of columns of z")
+    if parts <= 0 or inner % parts:
+        raise KernelError(f"gate_part_norm: {inner} values do not split into {parts} equal parts")
+    _f32_vector(weight, "weight", inner)
+    _row_facts(rows, row_slot=row_slot)
+    _check(_fn("ssm", "dryft_gate_part_norm")(_ptr(y), _ptr(z), z.stride(0), z_col, _ptr(weight), _ptr(row_slot), _ptr(out),
+                                              rows, inner, parts, float(eps), _float_flag(z, "z"), _stream()),
+           "gate_part_norm")
+
+
+# ------------------------------------------------------------------------------------------ gated delta rule
+DELTA_MAX_DIM = 256
+
+
+def delta_steps(qkv, q_col: int, k_col: int, v_col: int, gates, a_col: int, b_col: int, dt_bias, a_log, seq_slot, cu_rows,
+                q_len, n_seqs: int, state, out, n_heads: int, n_groups: int, key_dim: int, value_dim: int, q_scale: float,
+                unit_eps: float, write_state: bool) -> None:
+    """Per sequence and head, over the sequence's rows of the step in order, from ``state [slots, heads, key_dim,
+    value_dim]`` (float32): ``S <- g S``, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q`` with
+    ``g = exp(-exp(a_log) softplus(gates[:, a_col + h] + dt_bias))``, ``beta = sigmoid(gates[:, b_col + h])``, q and k
+    (``n_groups`` of them, runs of columns of ``qkv``) made unit vectors with ``unit_eps`` under the root, q times
+    ``q_scale``. ``out`` float32 ``[rows, heads * value_dim]`` (rows of sequences that sit out are not written)."""
+    _gpu(qkv, "qkv")
+    rows = qkv.shape[0]
+    if not (qkv.dim() == 2 and qkv.stride(1) == 1 and min(q_col, k_col, v_col) >= 0 and
+            max(q_col + n_groups * key_dim, k_col + n_groups * key_dim, v_col + n_heads * value_dim) <= qkv.shape[1]):
+        raise KernelError("delta_steps: q, k or v lie outside the columns of qkv")
+    _gpu(gates, "gates", torch.float32)
+    if not (gates.dim() == 2 and gates.shape[0] == rows and gates.stride(1) == 1 and min(a_col, b_col) >= 0 and
+            max(a_col, b_col) + n_heads <= gates.shape[1]):
+        raise KernelError("delta_steps: gates must be float32 [rows, columns] that hold a and b for every head")
+    _f32_vector(dt_bias, "dt_bias", n_heads)
+    _f32_vector(a_log, "a_log", n_heads)
+    _seq_facts(seq_slot, cu_rows, q_len, n_seqs)
+    _gpu(state, "state", torch.float32)
+    if not (state.dim() == 4 and state.shape[1:] == (n_heads, key_dim, value_dim) and state.is_contiguous()):
+        raise KernelError(f"delta_steps: state must be contiguous float32 [slots, {n_heads}, {key_dim}, {value_dim}]")
+    _gpu(out, "out", torch.float32)
+    if not (out.shape == (rows, n_heads * value_dim) and out.is_contiguous()):
+        raise KernelError("delta_steps: out must be contiguous float32 [rows, heads * value_dim]")
+    if not (0 < key_dim <= DELTA_MAX_DIM and n_groups > 0 and n_heads % n_groups == 0):
+        raise KernelError(f"delta_steps: keys of 1..{DELTA_MAX_DIM} features, heads a multiple of the key heads")
+    _check(_fn("delta", "dryft_delta_steps")(
+        _ptr(qkv), qkv.stride(0), q_col, k_col, v_col, _ptr(gates), gates.stride(0), a_col, b_col, _ptr(dt_bias),
+        _ptr(a_log), _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), _ptr(state), _ptr(out), n_seqs, n_heads, n_groups,
+        key_dim, value_dim, float(q_scale), float(unit_eps), int(bool(write_state)), _float_flag(qkv, "qkv"), _stream()),
+        "delta_steps")

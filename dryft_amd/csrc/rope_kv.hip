@@ -648,3 +648,116 @@ DRYFT_API int dryft_rope_pairs_kv(const void* proj, int64_t proj_stride, int q_c
                        v_col, row_slot, row_pos, (bf16_t*)v_pages, page_table, max_pages, n_rows, n_kv, v_dim);
   return DRYFT_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// A norm per head, a rotation over halves with float tables, and the append to the paged cache, for heads whose
+// keys and values may differ in width. Every q and k head is divided by its root mean square (eps inside the root)
+// and multiplied by a weight of head_dim entries (one for the queries, one for the keys; either may be absent, then
+// the head passes as it is). Of the first `rot` features of the normed head, feature i and feature i + rot/2 turn
+// together:
+//
+//   o[i] = x[i] c - x[i + rot/2] s,   o[i + rot/2] = x[i + rot/2] c + x[i] s,   c = cos_t[pos, i], s = sin_t[pos, i]
+//
+// and features from `rot` on pass. All of it is float arithmetic, rounded once on the way out. The row's q, k and v
+// start at columns q_col, k_col and v_col of `src`. One wave per head; the head waits in LDS between norm and turn.
+#define NRH_MAX_DIM 256
+
+template <typename T>
+__global__ __launch_bounds__(256) void norm_rope_half_kv_kernel(
+    const T* __restrict__ src_rows, int64_t src_stride, int q_col, int k_col, int v_col, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
+    const int* __restrict__ row_slot, const int* __restrict__ row_pos, T* __restrict__ q_out, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, const int* __restrict__ page_table, int max_pages, int write_kv, int n_heads, int n_kv,
+    int head_dim, int v_dim, int skip_v) {
+  __shared__ float held[4][NRH_MAX_DIM];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int64_t row = blockIdx.x;
+  const int job = blockIdx.y * 4 + wave;  // [0,nH): q heads; [nH,nH+nKV): k heads; then v heads
+  if (job >= n_heads + (skip_v ? 1 : 2) * n_kv) return;
+  const int slot = row_slot[row], pos = row_pos[row];
+  const bool is_q = job < n_heads, is_k = !is_q && job < n_heads + n_kv;
+  if (is_q) {
+    if (slot < 0) {
+      T* dst = q_out + (row * n_heads + job) * head_dim;
+      for (int i = lane; i < head_dim; i += WAVE) store_from_float(dst + i, 0.f);
+      return;
+    }
+  } else if (slot < 0 || !write_kv) {
+    return;
+  }
+  int page = 0, in_page = 0;
+  if (!is_q) {
+    page = page_of(page_table, max_pages, slot, pos);
+    in_page = pos % PAGE_TOKENS;
+    if (page < 0) return;  // no page: the host reserves one before the step; never write through a bad index
+  }
+  if (!is_q && !is_k) {
+    const int kvh = job - n_heads - n_kv;
+    const T* src = src_rows + row * src_stride + v_col + (int64_t)kvh * v_dim;
+    T* dst = v_pages + ((int64_t)page * n_kv + kvh) * v_dim * PAGE_TOKENS + value_column(in_page);
+    for (int i = lane; i < v_dim; i += WAVE) dst[(int64_t)i * PAGE_TOKENS] = src[i];
+    return;
+  }
+  const T* src = src_rows + row * src_stride + (is_q ? q_col + (int64_t)job * head_dim
+                                                     : k_col + (int64_t)(job - n_heads) * head_dim);
+  T* dst = is_q ? q_out + (row * n_heads + job) * head_dim
+                : k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + in_page) * head_dim;
+  const float* w = is_q ? q_w : k_w;
+  float* mine = held[wave];
+  float ss = 0.f;
+  for (int i = lane; i < head_dim; i += WAVE) {
+    const float v = load_as_float(src + i);
+    mine[i] = v;
+    ss += v * v;
+  }
+  const float inv = w != nullptr ? rsqrtf(wave_sum(ss) / (float)head_dim + eps) : 1.f;
+  const int half = rot / 2;
+  // each lane reads below what another lane of its wave wrote above
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  for (int i = lane; i < head_dim; i += WAVE) {
+    const float x = mine[i] * inv * (w != nullptr ? w[i] : 1.f);
+    float o = x;
+    if (i < rot) {
+      const int j = i < half ? i + half : i - half, f = i < half ? i : i - half;
+      const float other = mine[j] * inv * (w != nullptr ? w[j] : 1.f);
+      const float c = cos_t[(int64_t)pos * half + f], s = sin_t[(int64_t)pos * half + f];
+      o = i < half ? x * c - other * s : x * c + other * s;
+    }
+    store_from_float(dst + i, o);
+  }
+}
+
+DRYFT_API int dryft_norm_rope_half_kv(const void* src, int64_t src_stride, int q_col, int k_col, int v_col,
+                                      const float* q_w, const float* k_w, float eps, const float* cos_t,
+                                      const float* sin_t, int rot, const int* row_slot, const int* row_pos, void* q_out,
+                                      void* k_pages, void* v_pages, const int* page_table, int max_pages, int write_kv,
+                                      int n_rows, int n_heads, int n_kv, int head_dim, int v_dim, int is_f32,
+                                      hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (rot < 0 || rot % 2 || rot > head_dim || head_dim > NRH_MAX_DIM || n_kv <= 0 || q_out == nullptr) return -1;
+  // many rows: the values are transposed a tile of 64 rows at a time instead of 2 bytes at a time
+  const size_t v_lds = (size_t)v_dim * V_TILE_LD * (is_f32 ? 4 : 2);
+  const int skip_v = (write_kv && n_rows >= 32 && v_dim % 8 == 0 && v_col % 8 == 0 && src_stride % 8 == 0 &&
+                      (((uintptr_t)src | (uintptr_t)v_pages) & 15) == 0 && v_lds <= 64 * 1024) ? 1 : 0;
+  dim3 grid(n_rows, (n_heads + (skip_v ? 1 : 2) * n_kv + 3) / 4), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(norm_rope_half_kv_kernel<float>, grid, block, 0, stream, (const float*)src, src_stride, q_col,
+                       k_col, v_col, q_w, k_w, eps, cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out, (float*)k_pages,
+                       (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim, skip_v);
+  else
+    hipLaunchKernelGGL(norm_rope_half_kv_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)src, src_stride, q_col,
+                       k_col, v_col, q_w, k_w, eps, cos_t, sin_t, rot, row_slot, row_pos, (bf16_t*)q_out,
+                       (bf16_t*)k_pages, (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim,
+                       v_dim, skip_v);
+  int rc = DRYFT_LAUNCH_CHECK();
+  if (rc || !skip_v) return rc;
+  dim3 vgrid((n_rows + V_TILE_ROWS - 1) / V_TILE_ROWS, n_kv);
+  if (is_f32)
+    hipLaunchKernelGGL(v_tile_write_kernel<float>, vgrid, dim3(256), v_lds, stream, (const float*)src, src_stride,
+                       v_col, row_slot, row_pos, (float*)v_pages, page_table, max_pages, n_rows, n_kv, v_dim);
+  else
+    hipLaunchKernelGGL(v_tile_write_kernel<bf16_t>, vgrid, dim3(256), v_lds, stream, (const bf16_t*)src, src_stride,
+                       v_col, row_slot, row_pos, (bf16_t*)v_pages, page_table, max_pages, n_rows, n_kv, v_dim);
+  return DRYFT_LAUNCH_CHECK();
+}

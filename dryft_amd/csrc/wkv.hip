@@ -389,12 +389,13 @@ DRYFT_API int dryft_wkv_steps(const void* r, const void* k, const void* v, const
 template <typename T>
 __global__ __launch_bounds__(256) void wkv_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ gate,
                                                       const float* __restrict__ weight, T* __restrict__ out, int rows,
-                                                      int n_heads, int dim, float eps) {
+                                                      int n_heads, int dim, float eps, int64_t gate_stride) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t job = (int64_t)blockIdx.x * 4 + wave;
   if (job >= (int64_t)rows * n_heads) return;
   const int head = job % n_heads;
   const int64_t at = job * dim;
+  gate += (job / n_heads) * gate_stride + (int64_t)head * dim - at;      // the gate's rows may be a run of columns
   float ss = 0.f;
   for (int i = lane; i < dim; i += WAVE) { const float o = o_raw[at + i]; ss += o * o; }
   ss = wave_sum(ss);
@@ -406,15 +407,15 @@ __global__ __launch_bounds__(256) void wkv_out_kernel(const float* __restrict__ 
 }
 
 DRYFT_API int dryft_wkv_out(const float* o_raw, const void* gate, const float* weight, void* out, int rows, int n_heads,
-                            int dim, float eps, int is_f32, hipStream_t stream) {
+                            int dim, float eps, int64_t gate_stride, int is_f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   const int64_t jobs = (int64_t)rows * n_heads;
   dim3 grid((unsigned)((jobs + 3) / 4)), block(256);
   if (is_f32)
     hipLaunchKernelGGL(wkv_out_kernel<float>, grid, block, 0, stream, o_raw, (const float*)gate, weight, (float*)out, rows,
-                       n_heads, dim, eps);
+                       n_heads, dim, eps, gate_stride);
   else
     hipLaunchKernelGGL(wkv_out_kernel<bf16_t>, grid, block, 0, stream, o_raw, (const bf16_t*)gate, weight, (bf16_t*)out,
-                       rows, n_heads, dim, eps);
+                       rows, n_heads, dim, eps, gate_stride);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -12,7 +12,7 @@ import torch
 
 from ..config.plan import ModelPlan
 from ..parts import block_class, build_part
-from ..parts.base import Deferred, Partials, StepContext
+from ..parts.base import Deferred, Part, Partials, StepContext
 from ..weights.spec import TensorSpec
 from ..csrc import ops
 
@@ -99,8 +99,8 @@ class DecoderModel:
     def weight_bytes(self) -> int:
         seen, total = set(), 0
         for part, _ in self._bindings:
-            for v in vars(part).values():
-                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+            for v in _held_tensors(part):
+                if v.data_ptr() not in seen:
                     seen.add(v.data_ptr())
                     total += v.numel() * v.element_size()
         return total
@@ -111,8 +111,8 @@ class DecoderModel:
         for part, _ in self._bindings:
             if not part.reads_whole():
                 continue
-            for v in vars(part).values():
-                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+            for v in _held_tensors(part):
+                if v.data_ptr() not in seen:
                     seen.add(v.data_ptr())
                     total += v.numel() * v.element_size()
         return total
@@ -147,6 +147,7 @@ class DecoderModel:
         over nothing else. ``tap(i, stream)``, when given, is called after run ``i`` of the schedule with the residual
         stream as that run leaves it (float32, everything pending added): a way to look, not part of the step."""
         ctx.positions = self.positions
+        ctx.tokens = tokens
         x = self.embedding.forward(tokens)
         ctx.embedded = x
         pending = None
@@ -168,6 +169,16 @@ class DecoderModel:
     def logits(self, hidden: torch.Tensor, rows: torch.Tensor | None = None) -> torch.Tensor:
         """Float32 logits of hidden states that have been through the final norm (at ``rows`` of them; None: all)."""
         return self.head.forward(hidden if rows is None else _pick_rows(hidden, rows))
+
+
+def _held_tensors(part):
+    """The tensors a part holds, those of the parts it is made of included."""
+    for v in vars(part).values():
+        for u in (v.values() if isinstance(v, dict) else (v,)):
+            if isinstance(u, torch.Tensor):
+                yield u
+            elif isinstance(u, Part):
+                yield from _held_tensors(u)
 
 
 def _settled(x: torch.Tensor, pending) -> torch.Tensor:

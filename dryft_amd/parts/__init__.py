@@ -45,7 +45,7 @@ def build_part(spec) -> Part:
     return part_class(spec.kind)(**spec.args)
 
 
-from . import attention, block, embedding, experts, hyper, latent, mlp, norm, recurrent, rope, stream, wkv  # noqa: E402,F401  (register the built-in parts)
+from . import attention, block, delta, embedding, experts, hyper, latent, mlp, norm, parallel, recurrent, rope, ssm, stream, wkv  # noqa: E402,F401  (register the built-in parts)
 
 __all__ = ["Deferred", "StreamPart", "FeedForward", "HostBatch", "Mixer", "Norm", "Part", "Partials", "PositionEncoding", "StepContext", "matrix",
            "register_part", "register_block", "part_class", "block_class", "build_part"]

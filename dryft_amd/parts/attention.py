@@ -11,8 +11,11 @@ Options other designs use, all off by default: values of another width than the 
 capped score, ``s <- softcap * tanh(s / softcap)``; a sink per query head (tensor ``sink``), whose ``exp`` joins
 the softmax's denominator and nothing else; an output gate, the heads' outputs times ``sigmoid(W_g h)`` before
 the output projection (tensor ``g_proj``, fused into the q/k/v product); attention weights kept in float
-(``float_weights``); and, when the position encoding it names rotates neighbouring pairs
-(``PairRotaryPositions``), that rotation with float tables. Any of these takes the step down ``_forward_general``.
+(``float_weights``); biases on the q, k, v and output projections (``bias``); a short causal convolution over time on
+every channel of q, k and v right after the projection (``conv_taps``; the last ``taps - 1`` projected values of a
+sequence are then part of its state, beside its keys and values); and a position encoding with float tables, over
+neighbouring pairs (``PairRotaryPositions``) or over halves (``HalfRotaryPositions``; this one also after the per-head
+norms, in float). Any of these takes the step down ``_forward_general``.
 
 The part knows nothing of the model around it: sizes and constants are constructor arguments, the
 position encoding is looked up by name in the step context, and its storage is the cache line it
@@ -32,8 +35,9 @@ from ..limits import MATRIX_CORE_HEAD_STEP, MAX_HEAD_DIM
 from ..weights.spec import VECTOR
 from . import register_part
 from .base import Mixer, Partials, StepContext, matrix
+from .conv import conv_need, short_conv
 from .linear import linear
-from .rope import PairRotaryPositions
+from .rope import HalfRotaryPositions, PairRotaryPositions, RotaryPositions
 
 _RESIDENT_WORKGROUPS = 512     # of the split kernel: two per compute unit (its registers allow no more)
 _MAX_SPLITS = 32
@@ -41,12 +45,21 @@ _QKV_PARTIAL_ROWS = 256         # decoding steps of up to so many rows take the 
 _PROMPT_PARTIAL_ROWS = 256      # and so do prompt steps of at most so many rows
 
 
+def add_bias(delta, bias: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """``delta + bias`` per row in ``dtype``; ``delta`` is a tensor or ``Partials`` (added up on the way in)."""
+    data = delta.data if isinstance(delta, Partials) else delta
+    out = torch.empty(data.shape[-2:], dtype=dtype, device=data.device)
+    ops.stream_norm(None, (delta.data, delta.count) if isinstance(delta, Partials) else delta, None, None, bias, None, 0.0,
+                    None, out, dtype, plain_read=True)
+    return out
+
+
 class GQAAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: float | None = None, positions: str | None = None, rotary_dim: int | None = None,
                  window: int | None = None, scale: float | None = None, value_dim: int | None = None,
                  softcap: float | None = None, sink: bool = False, output_gate: bool = False,
-                 float_weights: bool = False):
+                 float_weights: bool = False, bias: bool = False, conv_taps: int | None = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} kv heads evenly")
         if not 0 < head_dim <= MAX_HEAD_DIM:
@@ -66,12 +79,14 @@ class GQAAttention(Mixer):
         self.has_sink, self.output_gate, self.float_weights = bool(sink), bool(output_gate), bool(float_weights)
         self.q_dim, self.kv_dim = self.n_heads * self.head_dim, self.n_kv * self.head_dim
         self.v_dim, self.o_dim = self.n_kv * self.value_dim, self.n_heads * self.value_dim
+        self.has_bias, self.conv_taps = bool(bias), int(conv_taps) if conv_taps else 0
+        if self.conv_taps > ops.CONV_MAX_TAPS:
+            raise ValueError(f"the convolution takes at most {ops.CONV_MAX_TAPS} taps, got {conv_taps}")
         self.extended = bool(self.value_dim != self.head_dim or self.softcap or self.has_sink or self.output_gate or
-                             self.float_weights)
-        if self.extended and self.qk_norm_eps is not None:
-            raise ValueError("per-head q/k norms are not combined with a capped score, a sink, an output gate or "
-                             "values of another width")
+                             self.float_weights or self.has_bias or self.conv_taps)
+        self.conv_channels = self.q_dim + self.kv_dim + self.v_dim
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.sink = None
+        self.in_bias = self.o_bias = self.conv_w = None
 
     def tensor_specs(self):
         specs = {"q_proj": matrix((self.q_dim, self.hidden)), "k_proj": matrix((self.kv_dim, self.hidden)),
@@ -83,6 +98,12 @@ class GQAAttention(Mixer):
         if self.qk_norm_eps is not None:
             specs["q_norm"] = ((self.head_dim,), VECTOR, "ones")
             specs["k_norm"] = ((self.head_dim,), VECTOR, "ones")
+        if self.has_bias:
+            specs.update({"q_bias": ((self.q_dim,), VECTOR, "normal"), "k_bias": ((self.kv_dim,), VECTOR, "normal"),
+                          "v_bias": ((self.v_dim,), VECTOR, "normal"), "o_bias": ((self.hidden,), VECTOR, "normal")})
+        if self.conv_taps:
+            specs.update({"q_conv": matrix((self.q_dim, self.conv_taps)), "k_conv": matrix((self.kv_dim, self.conv_taps)),
+                          "v_conv": matrix((self.v_dim, self.conv_taps))})
         return specs
 
     def load(self, tensors):
@@ -93,35 +114,58 @@ class GQAAttention(Mixer):
         self.w_o = tensors["o_proj"]
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = tensors["q_norm"], tensors["k_norm"]
-            if self.q_norm.dtype != self.k_norm.dtype:          # one kernel argument says how both are stored
-                self.q_norm, self.k_norm = self.q_norm.float(), self.k_norm.float()
+            if self.q_norm.dtype != self.k_norm.dtype or self.extended:   # one kernel argument says how both are stored
+                self.q_norm, self.k_norm = self.q_norm.float().contiguous(), self.k_norm.float().contiguous()
+        if self.has_bias:
+            self.in_bias = torch.cat([tensors[n].float() for n in ("q_bias", "k_bias", "v_bias")]).contiguous()
+            self.o_bias = tensors["o_bias"].float().contiguous()
+        if self.conv_taps:
+            self.conv_w = torch.cat([tensors[n].float() for n in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        elif self.has_bias:                   # the biases ride on a convolution of one tap
+            self.conv_w = torch.ones((self.conv_channels, 1), dtype=torch.float32, device=self.in_bias.device)
 
     def cache_need(self):
-        return KVNeed(self.n_kv, self.head_dim, self.window,
-                      self.value_dim if self.value_dim != self.head_dim else None)
+        kv = KVNeed(self.n_kv, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else None)
+        if self.conv_taps > 1:
+            return {"kv": kv, "tail": conv_need(self.conv_taps, self.conv_channels)}
+        return kv
 
     def kernel_modules(self, dtype):
         return ("gemm", "rope_kv", "attn_rows") + (("attn_mfma",) if dtype == torch.bfloat16 else ()) + \
-            (("activation",) if self.output_gate else ())
+            (("activation",) if self.output_gate else ()) + (("conv", "norm") if self.conv_taps or self.has_bias else ())
 
-    def _forward_general(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
-        """Every option, in float arithmetic on the kernel that takes one (row, head) a workgroup."""
+    def _forward_general(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
+        """Every option, in float arithmetic on the kernel that takes one (row, head) a workgroup. Returns the output
+        projection's result without its bias."""
         rows, H, G, D, Dv = h.shape[0], self.n_heads, self.n_kv, self.head_dim, self.value_dim
-        cos = sin = None
+        tail = line["tail"] if isinstance(line, dict) and "tail" in line else None
+        line = line["kv"] if isinstance(line, dict) else line
+        cos = sin = table = None
         rot = 0
         if self.positions:
             table = ctx.positions[self.positions]
-            if not isinstance(table, PairRotaryPositions):
-                raise NotImplementedError("the options of this attention go with a rotation over neighbouring pairs")
+            if not isinstance(table, (PairRotaryPositions, HalfRotaryPositions)):
+                raise NotImplementedError("the options of this attention go with a position encoding that has float tables")
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
             cos, sin, rot = table.cos, table.sin, table.dims
             if rot > D:
                 raise ValueError(f"the position encoding rotates {rot} features, a head has {D}")
         proj = linear(h, self.w_qkv)                                    # q | k | v | gate
+        src = proj
+        if self.conv_w is not None:
+            # biases and the short convolution: q | k | v as one run of channels, each with its own history
+            src = short_conv(proj, 0, self.conv_channels, self.conv_w, ctx, tail, writes_cache, in_bias=self.in_bias)
         q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
-        ops.rope_pairs_kv(proj, 0, self.q_dim, self.q_dim + self.kv_dim, cos, sin, rot, ctx.row_slot, ctx.row_pos, q,
-                          line.k, line.v, line.page_table, writes_cache, H, G, D, Dv)
+        if isinstance(table, PairRotaryPositions):
+            if self.qk_norm_eps is not None:
+                raise NotImplementedError("per-head q/k norms do not go with the rotation over neighbouring pairs")
+            ops.rope_pairs_kv(src, 0, self.q_dim, self.q_dim + self.kv_dim, cos, sin, rot, ctx.row_slot, ctx.row_pos, q,
+                              line.k, line.v, line.page_table, writes_cache, H, G, D, Dv)
+        else:
+            ops.norm_rope_half_kv(src, 0, self.q_dim, self.q_dim + self.kv_dim, self.q_norm, self.k_norm,
+                                  self.qk_norm_eps or 0.0, cos, sin, rot, ctx.row_slot, ctx.row_pos, q, line.k, line.v,
+                                  line.page_table, writes_cache, H, G, D, Dv)
         # bfloat16 on the matrix cores where they take the sizes (keys and values of one width, a multiple of 16);
         # float32, and the other sizes, on the kernel that takes one (row, head) a workgroup in float arithmetic
         matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0
@@ -153,9 +197,15 @@ class GQAAttention(Mixer):
             out = ops.sigmoid_gate(out, proj[:, g_col:g_col + self.o_dim], gated)
         return linear(out, self.w_o, allow_partials=True)
 
+    def forward_split(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
+        if self.has_bias:
+            return self._forward_general(h, ctx, line, writes_cache), self.o_bias
+        return self.forward(h, ctx, line, writes_cache), None
+
     def forward(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
-        if self.extended or (self.positions and isinstance(ctx.positions[self.positions], PairRotaryPositions)):
-            return self._forward_general(h, ctx, line, writes_cache)
+        if self.extended or (self.positions and not isinstance(ctx.positions[self.positions], RotaryPositions)):
+            out = self._forward_general(h, ctx, line, writes_cache)
+            return add_bias(out, self.o_bias, h.dtype) if self.has_bias else out
         rows = h.shape[0]
         # bfloat16 on the matrix cores where they take the head size; float32 and the other head sizes on the plain kernel
         matrix_cores = h.dtype == torch.bfloat16 and self.head_dim % MATRIX_CORE_HEAD_STEP == 0

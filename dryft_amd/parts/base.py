@@ -58,6 +58,7 @@ class StepContext:
     host: HostBatch | None = None
     positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
     embedded: torch.Tensor | None = None    # the embedding's output of this step's rows, for parts that come back to it
+    tokens: torch.Tensor | None = None      # the step's token ids (int32, a row each), for parts that look them up
     _tiles: dict[int, tuple[torch.Tensor, int]] = field(default_factory=dict, repr=False)
     _kept: dict[Any, torch.Tensor] = field(default_factory=dict, repr=False)
 
@@ -185,6 +186,11 @@ class Mixer(Part):
         """``h`` is ``[rows, hidden]``; returns a tensor of the same shape or ``Partials``. ``line`` is the storage
         ``cache_need`` asked for: a ``KVLine``, a ``StateLine``, None, or a dictionary of those under the same names."""
         raise NotImplementedError
+
+    def forward_split(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
+        """``(output without its last bias, that bias or None)``: for a consumer that adds the bias on its own way in
+        (a float32 vector of the output's width)."""
+        return self.forward(h, ctx, line, writes_cache), None
 
 
 class FeedForward(Part):

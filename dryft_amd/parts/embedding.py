@@ -1,6 +1,7 @@
 """Token embedding and output head.
 
-Embedding: a row gather without scaling (reference: engine/dryft_qwen3/model.py:132).
+Embedding: a row gather without scaling (reference: engine/dryft_qwen3/model.py:132); with ``scale`` the rows are
+multiplied by it and come out as float32, the start of a float32 residual stream.
 Head: ``logits = h @ W.T`` as float32. A tied head is a plan that gives the head the
 embedding's tensor name (weights.py:47-49): both parts then hold the same tensor. The reference keeps bfloat16 logits (model.py:186, 261); here the
 float accumulators are stored directly.
@@ -17,8 +18,9 @@ from .linear import linear
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float | None = None):
         self.vocab, self.hidden = int(vocab_size), int(hidden_size)
+        self.scale = float(scale) if scale is not None else None
         self.weight: torch.Tensor | None = None
 
     def tensor_specs(self):
@@ -34,6 +36,9 @@ class TokenEmbedding(Part):
         return False                      # a step gathers its rows' entries only
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        if self.scale is not None:
+            out = torch.empty((tokens.numel(), self.hidden), dtype=torch.float32, device=self.weight.device)
+            return ops.embed_scaled(tokens, self.weight, self.scale, out)
         out = torch.empty((tokens.numel(), self.hidden), dtype=self.weight.dtype, device=self.weight.device)
         return ops.embed_rows(tokens, self.weight, out)
 

@@ -8,6 +8,11 @@ weights ``s_e / (sum of the chosen s + 1e-20) * route_scale``. An expert is a cl
 ``down(g * sigmoid(alpha g) * (u + 1))`` with ``g = min(gate(h), limit)``, ``u = clamp(up(h), -limit, limit)``. The
 shared expert, of the same form with sizes of its own, runs for every row and is added times ``sigmoid(w_s . h)``.
 
+Other forms, by constructor arguments. ``router="table"``: no scores at all; an integer table ``[vocab, top]`` (the
+entries of a row differ) names each token id's experts, every one with weight ``1 / top`` (the step's token ids come
+with the step context). ``unit="silu"``: an expert is ``down(silu(gate(h)) * up(h))``, nothing clamped, and so is
+the shared expert, which is then added as it is.
+
 On the device throughout, so a step can be captured: the router picks, a small kernel sorts the (row, expert) pairs
 by expert and cuts each expert's run into tiles, and two grouped products walk the tiles (gate/up with the unit in
 the epilogue, then down); a last kernel adds each row's weighted outputs and the shared expert in a fixed order.
@@ -18,48 +23,71 @@ from __future__ import annotations
 import torch
 
 from ..csrc import ops
-from ..weights.spec import VECTOR
+from ..weights.spec import INT_TABLE, VECTOR
 from . import register_part
 from .base import FeedForward, Partials, matrix
 from .linear import linear
-from .mlp import ClampedGLU
+from .mlp import ClampedGLU, SwiGLU
 
 
 class RoutedExperts(FeedForward):
-    def __init__(self, hidden_size: int, experts: int, top: int, intermediate_size: int, limit: float,
+    def __init__(self, hidden_size: int, experts: int, top: int, intermediate_size: int, limit: float | None = None,
                  route_scale: float = 1.0, groups: tuple[int, int] | None = None,
-                 shared: tuple[int, float] | None = None, alpha: float = 1.702):
+                 shared: tuple | None = None, alpha: float = 1.702, router: str = "scores", unit: str = "clamped",
+                 vocab_size: int | None = None):
         self.hidden, self.n_experts, self.top, self.inter = int(hidden_size), int(experts), int(top), int(intermediate_size)
-        self.limit, self.alpha, self.route_scale = float(limit), float(alpha), float(route_scale)
+        if router not in ("scores", "table") or unit not in ("clamped", "silu"):
+            raise ValueError(f"router is 'scores' or 'table', unit 'clamped' or 'silu'; got {router!r}, {unit!r}")
+        if router == "table" and not vocab_size:
+            raise ValueError("a table router needs the vocabulary's size")
+        if unit == "clamped" and limit is None:
+            raise ValueError("the clamped unit needs its limit")
+        self.router, self.unit, self.vocab = router, unit, int(vocab_size or 0)
+        # the gated unit as the kernels take it: (limit, slope of the sigmoid, what is added to the up branch)
+        self.glu = (float(limit), float(alpha), 1.0) if unit == "clamped" else (float("inf"), 1.0, 0.0)
+        self.limit, self.alpha, self.route_scale = limit, float(alpha), float(route_scale)
         if not 1 <= self.top <= self.n_experts <= ops.MOE_MAX_EXPERTS:
             raise ValueError(f"1 <= top <= experts <= {ops.MOE_MAX_EXPERTS}, got top {top} of {experts}")
         self.groups = (int(groups[0]), int(groups[1])) if groups else (1, 1)
         count, keep = self.groups
         if self.n_experts % count or not 1 <= keep <= count or count > 64 or keep * (self.n_experts // count) < self.top:
             raise ValueError(f"{experts} experts in {count} groups of which {keep} are kept cannot give {top}")
-        self.shared = ClampedGLU(hidden_size, shared[0], shared[1], alpha) if shared else None
-        self.w_router = self.correction = self.w_gate_up = self.w_down = None
+        self.shared = None
+        if shared:
+            self.shared = ClampedGLU(hidden_size, shared[0], shared[1], alpha) if unit == "clamped" else \
+                SwiGLU(hidden_size, shared[0])
+        self.w_router = self.correction = self.w_gate_up = self.w_down = self.table = None
 
     def tensor_specs(self):
-        specs = {"router": matrix((self.n_experts, self.hidden)), "correction": ((self.n_experts,), VECTOR, "zeros")}
+        if self.router == "table":
+            specs = {"table": ((self.vocab, self.top), INT_TABLE, f"distinct<{self.n_experts}")}
+        else:
+            specs = {"router": matrix((self.n_experts, self.hidden)), "correction": ((self.n_experts,), VECTOR, "zeros")}
         for e in range(self.n_experts):
             specs[f"e{e}_gate"] = matrix((self.inter, self.hidden))
             specs[f"e{e}_up"] = matrix((self.inter, self.hidden))
             specs[f"e{e}_down"] = matrix((self.hidden, self.inter))
         if self.shared is not None:
             specs.update({"shared_" + k.split("_")[0]: v for k, v in self.shared.tensor_specs().items()})
-            specs["shared_weight"] = matrix((1, self.hidden))
+            if self.router == "scores":
+                specs["shared_weight"] = matrix((1, self.hidden))
         return specs
 
     def load(self, tensors):
         E = self.n_experts
         self.w_gate_up = torch.stack([torch.cat([tensors[f"e{e}_gate"], tensors[f"e{e}_up"]], dim=0) for e in range(E)]).contiguous()
         self.w_down = torch.stack([tensors[f"e{e}_down"] for e in range(E)]).contiguous()
-        self.correction = tensors["correction"].float().contiguous()
-        router = [tensors["router"]]
         if self.shared is not None:
             self.shared.compute_dtype = self.compute_dtype
             self.shared.load({k + "_proj": tensors["shared_" + k] for k in ("gate", "up", "down")})
+        if self.router == "table":
+            self.table = tensors["table"].to(torch.int32).contiguous()
+            if self.table.numel() and not (0 <= int(self.table.min()) and int(self.table.max()) < E):
+                raise ValueError(f"the experts' table names experts outside 0..{E - 1}")
+            return
+        self.correction = tensors["correction"].float().contiguous()
+        router = [tensors["router"]]
+        if self.shared is not None:
             router.append(tensors["shared_weight"])
         self.w_router = torch.cat(router, dim=0).contiguous()          # the shared expert's weight is one more logit
 
@@ -69,13 +97,17 @@ class RoutedExperts(FeedForward):
     def forward(self, h, ctx):
         rows, E, top = h.shape[0], self.n_experts, self.top
         dev = h.device
-        logits = linear(h, self.w_router, out_dtype=torch.float32)
         chosen = torch.empty((rows, top), dtype=torch.int32, device=dev)
         weights = torch.empty((rows, top), dtype=torch.float32, device=dev)
-        ops.moe_route(logits, self.correction, E, self.groups[0], self.groups[1], self.route_scale, chosen, weights)
+        logits = None
+        if self.router == "table":
+            ops.moe_table_route(ctx.tokens, self.table, E, chosen, weights)
+        else:
+            logits = linear(h, self.w_router, out_dtype=torch.float32)
+            ops.moe_route(logits, self.correction, E, self.groups[0], self.groups[1], self.route_scale, chosen, weights)
         plan = ops.moe_plan(chosen, E)
         act = torch.empty((rows * top, self.inter), dtype=h.dtype, device=dev)
-        ops.moe_products(h, self.w_gate_up, plan, act, top, glu=(self.limit, self.alpha))
+        ops.moe_products(h, self.w_gate_up, plan, act, top, glu=self.glu)
         y = torch.empty((rows * top, self.hidden), dtype=torch.float32, device=dev)
         ops.moe_products(act, self.w_down, plan, y, 0)
         shared = None
@@ -91,7 +123,9 @@ class RoutedExperts(FeedForward):
         return True
 
     def flops(self, rows, spans):
-        per_row = 2.0 * self.hidden * (self.n_experts + 1) + 6.0 * self.top * self.inter * self.hidden
+        per_row = 6.0 * self.top * self.inter * self.hidden
+        if self.router == "scores":
+            per_row += 2.0 * self.hidden * (self.n_experts + 1)
         if self.shared is not None:
             per_row += 6.0 * self.shared.inter * self.hidden
         return rows * per_row

@@ -87,22 +87,41 @@ class PairRotaryPositions(PositionEncoding):
 
 class HalfRotaryPositions(PositionEncoding):
     """Float32 tables for a rotation that pairs feature ``i`` with feature ``i + dims/2`` of the first ``dims``
-    features of a vector: ``cos``/``sin`` are ``[positions, dims / 2]`` of the angles ``p * base^(-2i / dims)``, formed
-    in float64 on the host and rounded once, whatever the activation dtype."""
+    features of a vector: ``cos``/``sin`` are ``[positions, dims / 2]`` of the angles ``p * f_i``,
+    ``f_i = base^(-2i / dims)``, formed in float64 on the host and rounded once, whatever the activation dtype.
 
-    def __init__(self, dims: int, base: float):
+    With ``scaling`` (``factor``, ``low``, ``high``, ``original``: the wavelength rule of Llama 3.1) a frequency whose
+    wavelength ``l = 2 pi / f`` is shorter than ``original / high`` stays, one whose wavelength is longer than
+    ``original / low`` becomes ``f / factor``, and between the two, with ``s = (original / l - low) / (high - low)``,
+    it becomes ``(1 - s) f / factor + s f``."""
+
+    def __init__(self, dims: int, base: float, scaling: dict | None = None):
         if dims % 2 or dims <= 0:
             raise ValueError(f"the rotated width must be even and positive, got {dims}")
         self.dims, self.base = int(dims), float(base)
+        self.scaling = dict(scaling) if scaling else None
+        if self.scaling:
+            missing = [k for k in ("factor", "low", "high", "original") if k not in self.scaling]
+            if missing or float(self.scaling["high"]) == float(self.scaling["low"]):
+                raise ValueError(f"frequency scaling needs factor, low, high (not equal) and original; got {self.scaling}")
         self.cos: torch.Tensor | None = None
         self.sin: torch.Tensor | None = None
         self.n_positions = 0
 
+    def frequencies(self) -> torch.Tensor:
+        f = self.base ** (-2.0 * torch.arange(self.dims // 2, dtype=torch.float64) / self.dims)
+        if not self.scaling:
+            return f
+        factor, low, high, original = (float(self.scaling[k]) for k in ("factor", "low", "high", "original"))
+        wave = 2.0 * math.pi / f
+        blend = ((original / wave - low) / (high - low))
+        mixed = (1.0 - blend) * f / factor + blend * f
+        return torch.where(wave < original / high, f, torch.where(wave > original / low, f / factor, mixed))
+
     def prepare(self, n_positions: int, dtype: torch.dtype, device) -> None:
         if self.cos is not None and n_positions <= self.n_positions:
             return
-        f = self.base ** (-2.0 * torch.arange(self.dims // 2, dtype=torch.float64) / self.dims)
-        angle = torch.arange(n_positions, dtype=torch.float64)[:, None] * f[None, :]
+        angle = torch.arange(n_positions, dtype=torch.float64)[:, None] * self.frequencies()[None, :]
         self.cos = angle.cos().to(torch.float32).to(device).contiguous()
         self.sin = angle.sin().to(torch.float32).to(device).contiguous()
         self.n_positions = n_positions

@@ -8,7 +8,10 @@ unadded (``Deferred``), and the next block's first kernel norms it, adds it, add
 due meanwhile, and norms the stream for its own first branch, in one launch.
 
 ``StreamRMSNorm``    the norm itself: ``x / sqrt(mean(x^2) + eps) * w`` in float, rounded once.
+``StreamLayerNorm``  the same with the mean taken off first: ``(x - mean) / sqrt(var + eps) * w``, no bias.
 ``SandwichBlock``    mixer and feed-forward, each between two norms; ``SandwichMixerBlock`` has the mixer alone.
+``PostNormBlock``    ``x <- x + norm(branch(x))``: the branches read the stream as it is, only their outputs are
+                     normed; ``PostNormMixerBlock`` has the mixer alone.
 ``PassEntry``        what a pass over a run of layers begins with: one learned vector per pass is added to the
                      stream, and from the second pass on the embedding's output once more.
 """
@@ -28,6 +31,8 @@ class StreamRMSNorm(Norm):
     the whole weight (a head's factor on its logits rides here). A stream of several copies ``[copies, rows, width]``
     (``parts/hyper.py``) is normed as the sum of its copies."""
 
+    centred = False           # does the norm take the mean off first (a layer norm without bias)?
+
     def __init__(self, size: int, eps: float, offset: float = 0.0, scale: float = 1.0):
         self.size, self.eps, self.offset, self.scale = int(size), float(eps), float(offset), float(scale)
         self.weight: torch.Tensor | None = None
@@ -45,7 +50,7 @@ class StreamRMSNorm(Norm):
         if x.dim() == 3:
             return self.add_forward(x, None, dtype)[1]
         y = torch.empty(x.shape, dtype=dtype or self.compute_dtype or x.dtype, device=x.device)
-        ops.stream_norm(x, None, None, None, None, self.weight, self.eps, None, y, y.dtype)
+        ops.stream_norm(x, None, None, None, None, self.weight, self.eps, None, y, y.dtype, centred=self.centred)
         return y
 
     def add_forward(self, res: torch.Tensor, delta, dtype: torch.dtype | None = None, in_place: bool = True):
@@ -60,8 +65,14 @@ class StreamRMSNorm(Norm):
         own = in_place and res.dtype == torch.float32 and res.is_contiguous()
         out = res if own else torch.empty(res.shape, dtype=torch.float32, device=res.device)
         y = torch.empty(res.shape, dtype=act, device=res.device)
-        _launch(res, pending, self.weight, self.eps, out, y, act)
+        _launch(res, pending, self.weight, self.eps, out, y, act, centred=self.centred)
         return out, y
+
+
+class StreamLayerNorm(StreamRMSNorm):
+    """``(x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * w`` in float, without a bias."""
+
+    centred = True
 
 
 def as_deferred(pending) -> Deferred:
@@ -79,14 +90,29 @@ def _activation_dtype(x: torch.Tensor, pending: Deferred) -> torch.dtype:
     return x.dtype
 
 
-def _launch(x, pending: Deferred, weight, eps, x_out, y, act) -> None:
+def _launch(x, pending: Deferred, weight, eps, x_out, y, act, centred: bool = False, plain_read: bool = False) -> None:
     delta = pending.delta
     if isinstance(delta, Partials):
         delta = (delta.data, delta.count)
     post = pending.norm.weight if pending.norm is not None else None
     if pending.norm is not None and pending.norm.eps != eps:
         raise ValueError("the norms around one residual sum differ in eps; one launch takes one")
-    ops.stream_norm(x, delta, post, pending.rows, pending.vector, weight, eps, x_out, y, act)
+    ops.stream_norm(x, delta, post, pending.rows, pending.vector, weight, eps, x_out, y, act,
+                    post_centred=bool(getattr(pending.norm, "centred", False)), centred=centred, plain_read=plain_read)
+
+
+def read_plain(x: torch.Tensor, pending, act: torch.dtype):
+    """``(stream, stream in act)`` after everything pending has entered the float32 stream ``x`` (updated in place):
+    for sublayers that read the stream as it is. Nothing pending and a float32 reader: the stream itself, no launch."""
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("a stream that is read as it is must be contiguous float32")
+    if pending is None and act == torch.float32:
+        return x, x
+    pending = as_deferred(pending)
+    y = torch.empty(x.shape, dtype=act, device=x.device)
+    eps = pending.norm.eps if pending.norm is not None else 0.0
+    _launch(x, pending, None, eps, x if pending.delta is not None else None, y, act, plain_read=True)
+    return x, y
 
 
 def settle(x: torch.Tensor, pending, eps: float = 0.0) -> torch.Tensor:
@@ -127,6 +153,33 @@ class SandwichMixerBlock(SandwichBlock):
     roles = ("mixer_norm", "mixer", "mixer_post_norm")
 
 
+class PostNormBlock:
+    """``x <- x + norm_a(mixer(x))``, then ``x <- x + norm_b(ffn(x))``: no norm in front of a sublayer. The stream is
+    float32 from the embedding on; as everywhere here a sublayer's output is handed on unadded and enters the stream
+    in the launch that also hands the next reader its rows."""
+
+    roles = ("mixer", "mixer_post_norm", "ffn", "ffn_post_norm")
+
+    def __init__(self, mixer: Mixer, mixer_post_norm: Norm, ffn: FeedForward | None = None,
+                 ffn_post_norm: Norm | None = None):
+        self.mixer, self.mixer_post_norm, self.ffn, self.ffn_post_norm = mixer, mixer_post_norm, ffn, ffn_post_norm
+
+    def parts(self):
+        return {role: getattr(self, role) for role in self.roles}
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache: bool):
+        x, h = read_plain(x, pending, ctx.dtype)
+        pending = Deferred(delta=self.mixer.forward(h, ctx, line, writes_cache), norm=self.mixer_post_norm)
+        if self.ffn is None:
+            return x, pending
+        x, h = read_plain(x, pending, ctx.dtype)
+        return x, Deferred(delta=self.ffn.forward(h, ctx), norm=self.ffn_post_norm)
+
+
+class PostNormMixerBlock(PostNormBlock):
+    roles = ("mixer", "mixer_post_norm")
+
+
 class PassEntry(StreamPart):
     """``steps [passes, width]``: pass ``t`` begins by adding ``steps[t]`` to every row of the stream, and every pass
     but the first (when ``readd_embedding``) by adding the embedding's output of the row once more."""
@@ -158,6 +211,9 @@ class PassEntry(StreamPart):
 
 
 register_part("stream_rmsnorm", StreamRMSNorm)
+register_part("stream_layernorm", StreamLayerNorm)
 register_part("pass_entry", PassEntry)
 register_block("sandwich", SandwichBlock)
 register_block("sandwich_mixer", SandwichMixerBlock)
+register_block("post_norm", PostNormBlock)
+register_block("post_norm_mixer", PostNormMixerBlock)

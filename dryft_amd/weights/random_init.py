@@ -31,7 +31,14 @@ def random_tensors(specs: Iterable[TensorSpec], seed: int, dtype: torch.dtype = 
     out: dict[str, torch.Tensor] = {}
     for s in specs:
         if s.role == INT_TABLE:
-            raise ValueError(f"{s.name}: integer tables have no random initialiser")
+            if not s.init.startswith("distinct<"):
+                raise ValueError(f"{s.name}: this integer table has no random initialiser")
+            bound = int(s.init[len("distinct<"):])          # each row: the first entries of a random order of 0..bound-1
+            if len(s.shape) != 2 or s.shape[1] > bound:
+                raise ValueError(f"{s.name}: {s.shape} cannot hold different integers below {bound} in every row")
+            order = torch.rand((s.shape[0], bound), generator=gen, dtype=torch.float32, device=device).argsort(dim=1)
+            out[s.name] = order[:, :s.shape[1]].to(torch.int32).contiguous()
+            continue
         if any(d < 0 for d in s.shape):
             raise ValueError(f"{s.name}: an extent that only a checkpoint decides has no random initialiser; "
                              "give it in the configuration")

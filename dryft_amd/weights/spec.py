@@ -14,10 +14,12 @@ class TensorSpec:
     name: str                      # name in the checkpoint
     shape: tuple[int, ...]
     role: str = MATRIX
-    init: str = "normal"           # random-weights mode: "normal", "ones", "zeros" or "eye" (a unit matrix)
+    # random-weights mode: "normal", "ones", "zeros", "eye" (a unit matrix), or for an integer table "distinct<n": every
+    # row holds different integers below n
+    init: str = "normal"
 
     def __post_init__(self):
         if self.role not in (MATRIX, VECTOR, INT_TABLE):
             raise ValueError(f"{self.name}: unknown role {self.role!r}")
-        if self.init not in ("normal", "ones", "zeros", "eye"):
+        if self.init not in ("normal", "ones", "zeros", "eye") and not self.init.startswith("distinct<"):
             raise ValueError(f"{self.name}: unknown init {self.init!r}")
