@@ -128,11 +128,13 @@ def compare_designs(args) -> int:
     return 0
 
 
-def compare_fetedra(args) -> int:
+def compare_fetedra(args, design: str = "fetedra", relative: str = "piralix") -> int:
     """``--design fetedra``: Fetedra at a few sizes with the widths of real models' layers beside the Piralix preset of
     the same width (the closest design the library has: mixed recurrent and attention layers on a float32 stream;
     the presets of a width hold about the same weight bytes); random weights, bfloat16, one prompt of
-    ``--prompt-len`` tokens and ``--batch`` sequences decoding. One JSON line."""
+    ``--prompt-len`` tokens and ``--batch`` sequences decoding. One JSON line. ``--design barilix`` does the same for
+    Barilix beside the Fetedra preset of the same width (recurrent and windowed-attention layers with experts on a
+    float32 stream, as many layers of the same widths)."""
     import torch
 
     from dryft_amd import Engine
@@ -144,13 +146,13 @@ def compare_fetedra(args) -> int:
         kw = dict(seed=args.seed, dtype="bfloat16", max_batch=args.batch, max_len=args.prompt_len + 2 * (args.steps + args.warmup) + 64,
                   use_graph=not args.no_graph)
         entry = {"preset": name, "width": raw["width"], "layers": len(raw["layers"])}
-        for key, cfg in (("fetedra", raw), ("piralix", load_preset(f"piralix-w{raw['width']}"))):
+        for key, cfg in ((design, raw), (relative, load_preset(f"{relative}-w{raw['width']}"))):
             engine = Engine(config=cfg, **kw)
             entry[key] = measure(engine, args.prompt_len, args.batch, args.steps, args.warmup, args.seed)
             del engine
             torch.cuda.empty_cache()
         sizes.append(entry)
-    print(json.dumps({"metric": "prefill and decode of Fetedra beside Piralix of equal width",
+    print(json.dumps({"metric": f"prefill and decode of {design.capitalize()} beside {relative.capitalize()} of equal width",
                       "dtype": "bf16", "data": "synthetic (random weights, uniform random token ids)",
                       "prompt_len": args.prompt_len, "batch": args.batch, "steps": args.steps, "warmup": args.warmup,
                       "graph": not args.no_graph, "sizes": sizes}))
@@ -160,9 +162,9 @@ def compare_fetedra(args) -> int:
 def main() -> int:
     global PROMPT, SLOT
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["piralix", "fetedra"],
+    ap.add_argument("--design", default=None, choices=["piralix", "fetedra", "barilix"],
                     help="instead of the default workload: that design beside its closest relative in the library at "
-                         "equal size (Piralix beside Qwen3, Fetedra beside Piralix; one JSON line)")
+                         "equal size (Piralix beside Qwen3, Fetedra beside Piralix, Barilix beside Fetedra; one JSON line)")
     ap.add_argument("--sizes", default=None, help="presets for --design (default: the design's presets)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
@@ -185,7 +187,10 @@ def main() -> int:
     SLOT = args.slot_len or max(SLOT, 2 * PROMPT)
     if args.design:
         args.sizes = args.sizes or {"piralix": "piralix-w1024,piralix-w2048,piralix-w2560",
-                                    "fetedra": "fetedra-w1024,fetedra-w2048"}[args.design]
+                                    "fetedra": "fetedra-w1024,fetedra-w2048",
+                                    "barilix": "barilix-w1024,barilix-w2048"}[args.design]
+        if args.design == "barilix":
+            return compare_fetedra(args, "barilix", "fetedra")
         return compare_fetedra(args) if args.design == "fetedra" else compare_designs(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (asked for {args.gpus}); this library has no multi-GPU path")

@@ -5,115 +5,155 @@
 //   S <- g_t S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t        (S is D x P per head)
 //
 // q and k (one per group of heads) arrive in the activation dtype from the short convolution and are made unit
-// vectors here, x / sqrt(sum(x^2) + 1e-6), q also times D^-1/2. The state is float32 in the state store and all of
-// the above is float arithmetic. A workgroup owns one (sequence, head, run of up to PT value columns) and walks the
-// sequence's rows of the step in order from the state the step before left. Thread (p, r) holds rows r, r + R, ... of
-// column p of S in registers (R = 256 / PT); the two sums over D of a token meet in LDS.
+// vectors here, x / sqrt(sum(x^2) + eps), q also times a factor. The state is float32 in the state store and all of
+// the above is float arithmetic.
+//
+// One wave owns one (sequence, head, run of value columns) and walks the sequence's rows of the step in order from
+// the state the step before left: a prompt, a portion of one and a single token are the same code. The walk is a
+// chain of dependent steps, so what counts is how short one step is: a column of S lives in the registers of LPC
+// neighbouring-by-stride lanes (D / LPC rows each, at most 64), so that both sums over D of a token are sums inside
+// a thread plus one or two lane exchanges, with no barrier and no trip through LDS. The token's k and q are the same
+// for every column: they wait in LDS, read as 16-byte broadcasts. Operands come in batches of eight tokens: while
+// the wave walks one batch, the next one's loads are in flight; the unit lengths (a sum over D per token) are taken
+// by four lanes a vector as the batch goes to LDS.
 #include "common.h"
 
-#define DELTA_THREADS 256
 #define DELTA_MAX_DIM 256
 #define DELTA_BATCH 8            // tokens whose operands are brought into LDS together
+#define DELTA_ROWS 64            // rows of a column a lane holds at most
 
 __device__ __forceinline__ float softplus_d(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-template <typename T, int PT>
-__global__ __launch_bounds__(DELTA_THREADS) void delta_steps_kernel(
+template <typename T, int LPC>
+__global__ __launch_bounds__(WAVE) void delta_steps_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, int q_col, int k_col, int v_col, const float* __restrict__ gates,
     int64_t gate_stride, int a_col, int b_col, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
     const int* __restrict__ seq_slot, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
     float* __restrict__ state, float* __restrict__ out, int H, int G, int D, int P, float q_scale, float unit_eps,
     int write_state) {
-  constexpr int R = DELTA_THREADS / PT, NS = DELTA_MAX_DIM / R, WAVES = DELTA_THREADS / WAVE;
-  __shared__ float sq[DELTA_BATCH][DELTA_MAX_DIM], sk[DELTA_BATCH][DELTA_MAX_DIM], sv[DELTA_BATCH][PT];
-  __shared__ float sg[DELTA_BATCH], sbeta[DELTA_BATCH];
-  __shared__ float red_k[R][PT], red_o[2][R][PT];
-  const int seq = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * PT;
+  constexpr int CW = WAVE / LPC;                       // columns a wave owns
+  constexpr int ROWS = DELTA_MAX_DIM / LPC < DELTA_ROWS ? DELTA_MAX_DIM / LPC : DELTA_ROWS;   // rows of a column a lane holds at most
+  constexpr int R4 = ROWS / 4;
+  constexpr int PER = DELTA_MAX_DIM / 4;               // values of a q or k vector one of its four lanes takes at most
+  // a vector in LDS: LPC runs of `rdp` floats (the rows of one lane), padded to a multiple of 4 with zeros
+  __shared__ __attribute__((aligned(16))) float sk[DELTA_BATCH][DELTA_MAX_DIM + 4 * LPC];
+  __shared__ __attribute__((aligned(16))) float sq[DELTA_BATCH][DELTA_MAX_DIM + 4 * LPC];
+  __shared__ float sv[DELTA_BATCH][CW], sg[DELTA_BATCH], sbeta[DELTA_BATCH];
+  const int seq = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * CW;
   const int slot = seq_slot[seq], rows = q_len[seq];
   if (slot < 0 || rows <= 0) return;
   const int64_t first = cu_rows[seq];
   const int group = head / (H / G);
-  const int p = threadIdx.x % PT, r = threadIdx.x / PT;
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const bool live = p0 + p < P;
-  const int cnt = (D - r + R - 1) / R;
-  float* mine = state + (((int64_t)slot * H + head) * D) * P + p0 + p;
-  float S[NS];
+  const int lane = threadIdx.x, col = lane % CW, sub = lane / CW;
+  const bool live = p0 + col < P;
+  const int rd = (D + LPC - 1) / LPC, rd4 = (rd + 3) / 4, rdp = 4 * rd4;     // rows a lane holds, in fours, padded
+  float* mine = state + (((int64_t)slot * H + head) * D) * P + p0 + col;
+  float S[ROWS];
 #pragma unroll
-  for (int i = 0; i < NS; ++i) S[i] = (live && i < cnt) ? mine[(int64_t)(r + i * R) * P] : 0.f;
+  for (int i = 0; i < ROWS; ++i) {
+    const int d = sub * rd + i;
+    S[i] = (live && i < rd && d < D) ? mine[(int64_t)d * P] : 0.f;
+  }
   const float rate = expf(a_log[head]), bias = dt_bias[head];
+  // the batch's loads: lane l takes part (l % 4) of vector (l / 4): token (l / 8), q or k ((l / 4) % 2)
+  const int vec = lane / 4, part = lane % 4, v_tok = vec >> 1, v_is_k = vec & 1;
+  const int per = (D + 3) / 4;                          // values of a vector a lane takes
+  float x[PER], vv[DELTA_BATCH * CW / WAVE], gate_a = 0.f, gate_b = 0.f;
+  auto fetch = [&](int t0) {
+    const int nb = min(DELTA_BATCH, rows - t0);
+    if (v_tok < nb) {
+      const T* src = qkv + (first + t0 + v_tok) * qkv_stride + (v_is_k ? k_col : q_col) + group * D + part * per;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) x[i] = (i < per && part * per + i < D) ? load_as_float(src + i) : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < DELTA_BATCH * CW / WAVE; ++j) {
+      const int idx = lane + j * WAVE, tt = idx / CW, pp = idx % CW;
+      vv[j] = (tt < nb && p0 + pp < P) ? load_as_float(qkv + (first + t0 + tt) * qkv_stride + v_col + head * P + p0 + pp) : 0.f;
+    }
+    if (lane < nb) {
+      const float* gr = gates + (first + t0 + lane) * gate_stride;
+      gate_a = gr[a_col + head];
+      gate_b = gr[b_col + head];
+    }
+  };
+  auto stage = [&](int t0) {
+    const int nb = min(DELTA_BATCH, rows - t0);
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) ss += x[i] * x[i];
+    ss += __shfl_xor(ss, 1, WAVE);
+    ss += __shfl_xor(ss, 2, WAVE);
+    if (v_tok < nb) {
+      const float inv = rsqrtf(ss + unit_eps) * (v_is_k ? 1.f : q_scale);
+      float* dst = v_is_k ? sk[v_tok] : sq[v_tok];
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int d = part * per + i;
+        if (i < per && d < D) dst[(d / rd) * rdp + d % rd] = x[i] * inv;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < DELTA_BATCH * CW / WAVE; ++j) {
+      const int idx = lane + j * WAVE;
+      sv[idx / CW][idx % CW] = vv[j];
+    }
+    if (lane < nb) {
+      sg[lane] = expf(-rate * softplus_d(gate_a + bias));
+      sbeta[lane] = 1.f / (1.f + expf(-gate_b));
+    }
+  };
+  // the padding of every run stays zero for good
+  for (int i = lane; i < DELTA_BATCH * (DELTA_MAX_DIM + 4 * LPC); i += WAVE) { (&sk[0][0])[i] = 0.f; (&sq[0][0])[i] = 0.f; }
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  fetch(0);
   for (int t0 = 0; t0 < rows; t0 += DELTA_BATCH) {
     const int nb = min(DELTA_BATCH, rows - t0);
-    __syncthreads();
-    // a wave takes a token's q, then its k: load, sum of squares, unit length
-    for (int job = wave; job < 2 * nb; job += WAVES) {
-      const int tt = job >> 1, is_k = job & 1;
-      const T* src = qkv + (first + t0 + tt) * qkv_stride + (is_k ? k_col : q_col) + group * D;
-      float x[DELTA_MAX_DIM / WAVE], ss = 0.f;
-#pragma unroll
-      for (int i = 0; i < DELTA_MAX_DIM / WAVE; ++i) {
-        const int d = lane + i * WAVE;
-        x[i] = d < D ? load_as_float(src + d) : 0.f;
-        ss += x[i] * x[i];
-      }
-      const float inv = rsqrtf(wave_sum(ss) + unit_eps) * (is_k ? 1.f : q_scale);
-      float* dst = is_k ? sk[tt] : sq[tt];
-#pragma unroll
-      for (int i = 0; i < DELTA_MAX_DIM / WAVE; ++i) {
-        const int d = lane + i * WAVE;
-        if (d < D) dst[d] = x[i] * inv;
-      }
-    }
-    for (int i = threadIdx.x; i < nb * PT; i += DELTA_THREADS) {
-      const int tt = i / PT, pp = i % PT;
-      sv[tt][pp] = p0 + pp < P ? load_as_float(qkv + (first + t0 + tt) * qkv_stride + v_col + head * P + p0 + pp) : 0.f;
-    }
-    if (threadIdx.x < nb) {
-      const float* gr = gates + (first + t0 + threadIdx.x) * gate_stride;
-      sg[threadIdx.x] = expf(-rate * softplus_d(gr[a_col + head] + bias));
-      sbeta[threadIdx.x] = 1.f / (1.f + expf(-gr[b_col + head]));
-    }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");      // the walk over the batch before is done with LDS
+    __builtin_amdgcn_wave_barrier();
+    stage(t0);
+    if (t0 + DELTA_BATCH < rows) fetch(t0 + DELTA_BATCH);
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+    __builtin_amdgcn_wave_barrier();
     for (int tt = 0; tt < nb; ++tt) {
-      const float g = sg[tt];
+      const float g = sg[tt], beta = sbeta[tt], v = sv[tt][col];
+      const vf4* kp = (const vf4*)(sk[tt] + sub * rdp);
+      const vf4* qp = (const vf4*)(sq[tt] + sub * rdp);
       float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < NS; ++i) {
-        if (i < cnt) {
-          S[i] *= g;
-          acc += S[i] * sk[tt][r + i * R];
+      for (int i = 0; i < R4; ++i) {
+        if (i < rd4) {
+          const vf4 kk = kp[i];
+          acc += S[4 * i] * kk[0] + S[4 * i + 1] * kk[1] + S[4 * i + 2] * kk[2] + S[4 * i + 3] * kk[3];
         }
       }
-      red_k[r][p] = acc;
-      __syncthreads();
-      float ks = 0.f;
 #pragma unroll
-      for (int k = 0; k < R; ++k) ks += red_k[k][p];
-      const float u = sbeta[tt] * (sv[tt][p] - ks);
-      acc = 0.f;
+      for (int o = CW; o < WAVE; o <<= 1) acc += __shfl_xor(acc, o, WAVE);
+      const float u = beta * (v - g * acc);
+      float res = 0.f;
 #pragma unroll
-      for (int i = 0; i < NS; ++i) {
-        if (i < cnt) {
-          const int d = r + i * R;
-          S[i] += sk[tt][d] * u;
-          acc += S[i] * sq[tt][d];
+      for (int i = 0; i < R4; ++i) {
+        if (i < rd4) {
+          const vf4 kk = kp[i], qq = qp[i];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            S[4 * i + j] = g * S[4 * i + j] + kk[j] * u;
+            res += S[4 * i + j] * qq[j];
+          }
         }
       }
-      const int par = tt & 1;
-      red_o[par][r][p] = acc;
-      __syncthreads();
-      if (r == 0 && live) {
-        float sum = 0.f;
 #pragma unroll
-        for (int k = 0; k < R; ++k) sum += red_o[par][k][p];
-        out[(first + t0 + tt) * (int64_t)(H * P) + head * P + p0 + p] = sum;
-      }
+      for (int o = CW; o < WAVE; o <<= 1) res += __shfl_xor(res, o, WAVE);
+      if (sub == 0 && live) out[(first + t0 + tt) * (int64_t)(H * P) + head * P + p0 + col] = res;
     }
   }
   if (write_state && live) {
 #pragma unroll
-    for (int i = 0; i < NS; ++i)
-      if (i < cnt) mine[(int64_t)(r + i * R) * P] = S[i];
+    for (int i = 0; i < ROWS; ++i) {
+      const int d = sub * rd + i;
+      if (i < rd && d < D) mine[(int64_t)d * P] = S[i];
+    }
   }
 }
 
@@ -126,14 +166,17 @@ DRYFT_API int dryft_delta_steps(const void* qkv, int64_t qkv_stride, int q_col, 
                                 int is_f32, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || D > DELTA_MAX_DIM || P <= 0) return -1;
-#define DELTA_LAUNCH(TT, PTV)                                                                                          \
-  hipLaunchKernelGGL((delta_steps_kernel<TT, PTV>), dim3(n_seqs, H, (P + PTV - 1) / PTV), dim3(DELTA_THREADS), 0,     \
+#define DELTA_LAUNCH(TT, L)                                                                                           \
+  hipLaunchKernelGGL((delta_steps_kernel<TT, L>), dim3(n_seqs, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0,   \
                      stream, (const TT*)qkv, qkv_stride, q_col, k_col, v_col, gates, gate_stride, a_col, b_col, dt_bias, \
                      a_log, seq_slot, cu_rows, q_len, state, out, H, G, D, P, q_scale, unit_eps, write_state)
+  // lanes a column: as few as hold its rows (64 each), and no more columns a wave than the head has
+  int lpc = D > 128 ? 4 : (D > 64 ? 2 : 1);
+  while (lpc < 4 && WAVE / lpc > P && WAVE / (2 * lpc) >= 8) lpc *= 2;
   if (is_f32) {
-    if (P > 32) DELTA_LAUNCH(float, 64); else if (P > 16) DELTA_LAUNCH(float, 32); else DELTA_LAUNCH(float, 16);
+    if (lpc == 4) DELTA_LAUNCH(float, 4); else if (lpc == 2) DELTA_LAUNCH(float, 2); else DELTA_LAUNCH(float, 1);
   } else {
-    if (P > 32) DELTA_LAUNCH(bf16_t, 64); else if (P > 16) DELTA_LAUNCH(bf16_t, 32); else DELTA_LAUNCH(bf16_t, 16);
+    if (lpc == 4) DELTA_LAUNCH(bf16_t, 4); else if (lpc == 2) DELTA_LAUNCH(bf16_t, 2); else DELTA_LAUNCH(bf16_t, 1);
   }
 #undef DELTA_LAUNCH
   return DRYFT_LAUNCH_CHECK();
