@@ -73,6 +73,23 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum over groups of N neighbouring lanes (N a power of two up to 16, groups aligned to N): every lane of a group gets
+// the group's sum. Lane exchanges inside a row of 16 lanes are data-parallel-primitive moves (no trip through LDS):
+// the neighbour, the other pair of a quad, the mirrored half row, the mirrored row.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int N>
+__device__ __forceinline__ float lanes_sum(float v) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "groups of 1, 2, 4, 8 or 16 lanes");
+  if (N >= 2) v += dpp_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  if (N >= 4) v += dpp_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if (N >= 8) v += dpp_move<0x141>(v);     // row_half_mirror: lane i of a half row takes lane 7 - i
+  if (N >= 16) v += dpp_move<0x140>(v);    // row_mirror: lane i of a row takes lane 15 - i
+  return v;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));

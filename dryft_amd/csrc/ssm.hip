@@ -8,10 +8,11 @@
 // activation dtype (the output of the short convolution). One wave owns one (sequence, head, run of value columns)
 // and walks the sequence's rows of the step in order from the state the step before left: a prompt, a portion of
 // one and a single token are the same code. The walk is a chain of dependent steps: a column of S lives in the
-// registers of LPC lanes (N / LPC rows each, at most 64), so that a token's sum over N is a sum inside a thread plus
-// one or two lane exchanges, with no barrier. B and C of a token are the same for every column: they wait in LDS,
-// read as 16-byte broadcasts. Operands come in batches of eight tokens; the next batch's loads are in flight while
-// the wave walks the current one.
+// registers of LPC neighbouring lanes (N / LPC rows each, at most 64), so that a token's sum over N is a sum inside
+// a thread plus LPC's worth of lane exchanges inside a row of lanes, with no barrier. The host takes as many lanes
+// a column as still leave every lane eight rows and the chip a wave per SIMD. B and C of a token are the same for
+// every column: they wait in LDS, one run per lane of a column (runs a bank apart), read 16 bytes at a time.
+// Operands come in batches of eight tokens; the next batch's loads are in flight while the wave walks this one.
 #include "common.h"
 
 #define SSM_MAX_STATE 256
@@ -25,23 +26,25 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     const T* __restrict__ xbc, int64_t xbc_stride, int x_col, int b_col, int c_col, const float* __restrict__ dt_raw,
     int64_t dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
     const int* __restrict__ seq_slot, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
-    float* __restrict__ state, float* __restrict__ y, int H, int P, int N, int G, int write_state) {
+    float* __restrict__ state, float* __restrict__ y, int H, int P, int N, int G, int write_state, int vec8) {
   constexpr int CW = WAVE / LPC;                       // columns a wave owns
-  constexpr int ROWS = SSM_MAX_STATE / LPC < SSM_ROWS ? SSM_MAX_STATE / LPC : SSM_ROWS;   // rows of a column a lane holds at most
+  constexpr int ROWS = SSM_MAX_STATE / LPC < SSM_ROWS ? SSM_MAX_STATE / LPC : SSM_ROWS;
   constexpr int R4 = ROWS / 4;
   constexpr int PER = SSM_MAX_STATE / 4;               // values of a B or C vector one of its four lanes takes at most
-  // a vector in LDS: LPC runs of `rdp` floats (the rows of one lane), padded to a multiple of 4 with zeros
-  __shared__ __attribute__((aligned(16))) float sB[SSM_BATCH][SSM_MAX_STATE + 4 * LPC];
-  __shared__ __attribute__((aligned(16))) float sC[SSM_BATCH][SSM_MAX_STATE + 4 * LPC];
+  constexpr int VN = (SSM_BATCH * CW + WAVE - 1) / WAVE;
+  // a vector in LDS: LPC runs (the rows of one lane each), a run padded with zeros to a multiple of 4 floats and
+  // followed by 4 more so that neighbouring runs start in different banks
+  __shared__ __attribute__((aligned(16))) float sB[SSM_BATCH][SSM_MAX_STATE + 8 * LPC];
+  __shared__ __attribute__((aligned(16))) float sC[SSM_BATCH][SSM_MAX_STATE + 8 * LPC];
   __shared__ float sx[SSM_BATCH][CW], sdt[SSM_BATCH], sa[SSM_BATCH];
   const int seq = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * CW;
   const int slot = seq_slot[seq], rows = q_len[seq];
   if (slot < 0 || rows <= 0) return;
   const int64_t first = cu_rows[seq];
   const int group = head / (H / G);
-  const int lane = threadIdx.x, col = lane % CW, sub = lane / CW;
+  const int lane = threadIdx.x, sub = lane % LPC, col = lane / LPC;
   const bool live = p0 + col < P;
-  const int rd = (N + LPC - 1) / LPC, rd4 = (rd + 3) / 4, rdp = 4 * rd4;
+  const int rd = (N + LPC - 1) / LPC, rd4 = (rd + 3) / 4, run = 4 * rd4 + 4;
   float* mine = state + (((int64_t)slot * H + head) * N) * P + p0 + col;
   float S[ROWS];
 #pragma unroll
@@ -52,17 +55,28 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
   const float rate = expf(a_log[head]), bias = dt_bias[head], skip = d_skip[head];
   // the batch's loads: lane l takes part (l % 4) of vector (l / 4): token (l / 8), B or C ((l / 4) % 2)
   const int vec = lane / 4, part = lane % 4, v_tok = vec >> 1, v_is_c = vec & 1;
-  const int per = (N + 3) / 4;
-  float bc[PER], xv[SSM_BATCH * CW / WAVE], dtr = 0.f;
+  const int per = vec8 ? N / 4 : (N + 3) / 4;
+  const int run0 = (part * per) / rd, off0 = (part * per) % rd;   // where its first value goes
+  float bc[PER], xv[VN], dtr = 0.f;
   auto fetch = [&](int t0) {
     const int nb = min(SSM_BATCH, rows - t0);
     if (v_tok < nb) {
       const T* src = xbc + (first + t0 + v_tok) * xbc_stride + (v_is_c ? c_col : b_col) + group * N + part * per;
+      if (vec8) {
 #pragma unroll
-      for (int i = 0; i < PER; ++i) bc[i] = (i < per && part * per + i < N) ? load_as_float(src + i) : 0.f;
+        for (int i = 0; i < PER / 8; ++i) {
+          float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          if (8 * i < per) load8_as_float(src + 8 * i, t);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) bc[8 * i + j] = t[j];
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) bc[i] = (i < per && part * per + i < N) ? load_as_float(src + i) : 0.f;
+      }
     }
 #pragma unroll
-    for (int j = 0; j < SSM_BATCH * CW / WAVE; ++j) {
+    for (int j = 0; j < VN; ++j) {
       const int idx = lane + j * WAVE, tt = idx / CW, pp = idx % CW;
       xv[j] = (tt < nb && p0 + pp < P) ? load_as_float(xbc + (first + t0 + tt) * xbc_stride + x_col + head * P + p0 + pp) : 0.f;
     }
@@ -72,16 +86,17 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     const int nb = min(SSM_BATCH, rows - t0);
     if (v_tok < nb) {
       float* dst = v_is_c ? sC[v_tok] : sB[v_tok];
+      int r = run0, o = off0;
 #pragma unroll
       for (int i = 0; i < PER; ++i) {
-        const int n = part * per + i;
-        if (i < per && n < N) dst[(n / rd) * rdp + n % rd] = bc[i];
+        if (i < per && part * per + i < N) dst[r * run + o] = bc[i];
+        if (++o == rd) { o = 0; ++r; }
       }
     }
 #pragma unroll
-    for (int j = 0; j < SSM_BATCH * CW / WAVE; ++j) {
+    for (int j = 0; j < VN; ++j) {
       const int idx = lane + j * WAVE;
-      sx[idx / CW][idx % CW] = xv[j];
+      if (idx < SSM_BATCH * CW) sx[idx / CW][idx % CW] = xv[j];
     }
     if (lane < nb) {
       const float dt = softplus_f(dtr + bias);
@@ -89,23 +104,24 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
       sa[lane] = expf(-rate * dt);
     }
   };
-  // the padding of every run stays zero for good
-  for (int i = lane; i < SSM_BATCH * (SSM_MAX_STATE + 4 * LPC); i += WAVE) { (&sB[0][0])[i] = 0.f; (&sC[0][0])[i] = 0.f; }
-  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
-  __builtin_amdgcn_wave_barrier();
+  if (4 * rd4 != rd || rd * LPC != N) {                // what pads the runs stays zero for good
+    for (int i = lane; i < SSM_BATCH * (SSM_MAX_STATE + 8 * LPC); i += WAVE) { (&sB[0][0])[i] = 0.f; (&sC[0][0])[i] = 0.f; }
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
   fetch(0);
   for (int t0 = 0; t0 < rows; t0 += SSM_BATCH) {
     const int nb = min(SSM_BATCH, rows - t0);
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");      // the walk over the batch before is done with LDS
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");      // one wave: order only, the loads in flight stay in flight
     __builtin_amdgcn_wave_barrier();
     stage(t0);
     if (t0 + SSM_BATCH < rows) fetch(t0 + SSM_BATCH);
-    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
     for (int tt = 0; tt < nb; ++tt) {
       const float a = sa[tt], x = sx[tt][col], dtx = sdt[tt] * x;
-      const vf4* bp = (const vf4*)(sB[tt] + sub * rdp);
-      const vf4* cp = (const vf4*)(sC[tt] + sub * rdp);
+      const vf4* bp = (const vf4*)(sB[tt] + sub * run);
+      const vf4* cp = (const vf4*)(sC[tt] + sub * run);
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < R4; ++i) {
@@ -118,8 +134,7 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
           }
         }
       }
-#pragma unroll
-      for (int o = CW; o < WAVE; o <<= 1) acc += __shfl_xor(acc, o, WAVE);
+      acc = lanes_sum<LPC>(acc);
       if (sub == 0 && live) y[(first + t0 + tt) * (int64_t)(H * P) + head * P + p0 + col] = acc + skip * x;
     }
   }
@@ -164,24 +179,42 @@ __global__ __launch_bounds__(256) void gate_part_norm_kernel(const float* __rest
 
 DRYFT_API int dryft_ssm_max_state() { return SSM_MAX_STATE; }
 
+// Lanes a column: as few as hold its rows (64 each), then more while every lane keeps eight rows or more and the
+// launch stays within a wave per SIMD of the chip.
+static int lanes_per_column(int rows_of_state, int n_seqs, int heads, int columns) {
+  int lpc = rows_of_state > 128 ? 4 : (rows_of_state > 64 ? 2 : 1);
+  while (lpc < 16) {
+    const int next = 2 * lpc, cw = WAVE / next;
+    if ((rows_of_state + next - 1) / next < 8) break;
+    if ((int64_t)n_seqs * heads * ((columns + cw - 1) / cw) > 1024 && cw < columns) break;
+    lpc = next;
+  }
+  return lpc;
+}
+
 DRYFT_API int dryft_ssm_scan(const void* xbc, int64_t xbc_stride, int x_col, int b_col, int c_col, const float* dt_raw,
                              int64_t dt_stride, const float* dt_bias, const float* a_log, const float* d_skip,
                              const int* seq_slot, const int* cu_rows, const int* q_len, float* state, float* y, int n_seqs,
                              int H, int P, int N, int G, int write_state, int is_f32, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   if (H <= 0 || P <= 0 || N <= 0 || N > SSM_MAX_STATE || G <= 0 || H % G) return -1;
+  // 16-byte loads of B and C: a lane's quarter of a vector in whole pieces of 8 values, at aligned addresses
+  const int vec8 = (N % 32 == 0 && b_col % 8 == 0 && c_col % 8 == 0 && xbc_stride % 8 == 0 && ((uintptr_t)xbc & 15) == 0) ? 1 : 0;
 #define SSM_LAUNCH(TT, L)                                                                                             \
   hipLaunchKernelGGL((ssm_scan_kernel<TT, L>), dim3(n_seqs, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0, stream, \
                      (const TT*)xbc, xbc_stride, x_col, b_col, c_col, dt_raw, dt_stride, dt_bias, a_log, d_skip,      \
-                     seq_slot, cu_rows, q_len, state, y, H, P, N, G, write_state)
-  // lanes a column: as few as hold its rows (64 each), and no more columns a wave than the head has
-  int lpc = N > 128 ? 4 : (N > 64 ? 2 : 1);
-  while (lpc < 4 && WAVE / lpc > P && WAVE / (2 * lpc) >= 8) lpc *= 2;
-  if (is_f32) {
-    if (lpc == 4) SSM_LAUNCH(float, 4); else if (lpc == 2) SSM_LAUNCH(float, 2); else SSM_LAUNCH(float, 1);
-  } else {
-    if (lpc == 4) SSM_LAUNCH(bf16_t, 4); else if (lpc == 2) SSM_LAUNCH(bf16_t, 2); else SSM_LAUNCH(bf16_t, 1);
+                     seq_slot, cu_rows, q_len, state, y, H, P, N, G, write_state, vec8)
+#define SSM_PICK(TT)                                                                                                  \
+  switch (lpc) {                                                                                                      \
+    case 16: SSM_LAUNCH(TT, 16); break;                                                                               \
+    case 8: SSM_LAUNCH(TT, 8); break;                                                                                 \
+    case 4: SSM_LAUNCH(TT, 4); break;                                                                                 \
+    case 2: SSM_LAUNCH(TT, 2); break;                                                                                 \
+    default: SSM_LAUNCH(TT, 1);                                                                                       \
   }
+  const int lpc = lanes_per_column(N, n_seqs, H, P);
+  if (is_f32) { SSM_PICK(float) } else { SSM_PICK(bf16_t) }
+#undef SSM_PICK
 #undef SSM_LAUNCH
   return DRYFT_LAUNCH_CHECK();
 }
