@@ -25,13 +25,24 @@
 
 __device__ __forceinline__ float softplus_d(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-template <typename T, int LPC>
+//
+// Long prompts are cut into segments of `seg_rows` rows that run side by side (MODE 1, then the carry kernel, then
+// MODE 2; MODE 0 walks a whole sequence). A token maps every column of the state alike, c -> g (I - beta k k^T) c +
+// beta k v_c, so a segment's effect is S_out = A S_in + L with A (D x D) the product of its tokens' maps and L the
+// state it reaches from zero. MODE 1 computes both for every segment but a sequence's last, without read-outs: L
+// by the walk from zero, and A by the same walk, with values of zero, over the D columns of the unit matrix (the
+// waves of the grid behind those of the value columns). The carry kernel walks a sequence's segments and leaves each
+// the state that enters it; MODE 2 starts every segment from that state and writes its read-outs, and a sequence's
+// last segment writes the state back. Segment x of the step belongs to the sequence s with seg_cu[s] <= x <
+// seg_cu[s + 1] (prefix sums over the sequences; one that sits out has none).
+template <typename T, int LPC, int MODE>
 __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, int q_col, int k_col, int v_col, const float* __restrict__ gates,
     int64_t gate_stride, int a_col, int b_col, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
     const int* __restrict__ seq_slot, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
     float* __restrict__ state, float* __restrict__ out, int H, int G, int D, int P, float q_scale, float unit_eps,
-    int write_state, int vec8) {
+    int write_state, int vec8, const int* __restrict__ seg_cu, int n_seqs, int seg_rows, float* __restrict__ seg_state,
+    float* __restrict__ seg_trans) {
   constexpr int CW = WAVE / LPC;                       // columns a wave owns
   constexpr int ROWS = DELTA_MAX_DIM / LPC < DELTA_ROWS ? DELTA_MAX_DIM / LPC : DELTA_ROWS;
   constexpr int R4 = ROWS / 4;
@@ -42,20 +53,38 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
   __shared__ __attribute__((aligned(16))) float sk[DELTA_BATCH][DELTA_MAX_DIM + 8 * LPC];
   __shared__ __attribute__((aligned(16))) float sq[DELTA_BATCH][DELTA_MAX_DIM + 8 * LPC];
   __shared__ float sv[DELTA_BATCH][CW], sg[DELTA_BATCH], sbeta[DELTA_BATCH];
-  const int seq = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * CW;
-  const int slot = seq_slot[seq], rows = q_len[seq];
+  const int head = blockIdx.y, z_values = (P + CW - 1) / CW;
+  const bool unit = MODE == 1 && (int)blockIdx.z >= z_values;      // this wave walks columns of the unit matrix
+  const int p0 = (unit ? blockIdx.z - z_values : blockIdx.z) * CW;
+  int seq = blockIdx.x, seg = 0, n_segs = 1;
+  if (MODE != 0) {
+    if ((int)blockIdx.x >= seg_cu[n_seqs]) return;
+    seq = 0;
+    while (seg_cu[seq + 1] <= (int)blockIdx.x) ++seq;
+    seg = blockIdx.x - seg_cu[seq];
+    n_segs = seg_cu[seq + 1] - seg_cu[seq];
+    if (MODE == 1 && seg == n_segs - 1) return;                   // nobody needs the last segment's summary
+  }
+  const int slot = seq_slot[seq];
+  const int rows = MODE == 0 ? q_len[seq] : min(seg_rows, q_len[seq] - seg * seg_rows);
   if (slot < 0 || rows <= 0) return;
-  const int64_t first = cu_rows[seq];
+  const int64_t first = cu_rows[seq] + (MODE == 0 ? 0 : seg * seg_rows);
   const int group = head / (H / G);
   const int lane = threadIdx.x, sub = lane % LPC, col = lane / LPC;
-  const bool live = p0 + col < P;
+  const int width = unit ? D : P;                                  // columns of what this wave walks
+  const bool live = p0 + col < width;
   const int rd = (D + LPC - 1) / LPC, rd4 = (rd + 3) / 4, run = 4 * rd4 + 4;    // rows a lane holds, in fours, a run in LDS
   float* mine = state + (((int64_t)slot * H + head) * D) * P + p0 + col;
+  float* seg_mine = MODE == 0 ? nullptr
+                    : unit    ? seg_trans + (((int64_t)blockIdx.x * H + head) * D + p0 + col) * D
+                              : seg_state + (((int64_t)blockIdx.x * H + head) * D) * P + p0 + col;
+  const float* from = MODE == 2 ? seg_mine : mine;
   float S[ROWS];
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) {
     const int d = sub * rd + i;
-    S[i] = (live && i < rd && d < D) ? mine[(int64_t)d * P] : 0.f;
+    if (MODE == 1) S[i] = (unit && live && i < rd && d == p0 + col) ? 1.f : 0.f;
+    else S[i] = (live && i < rd && d < D) ? from[(int64_t)d * P] : 0.f;
   }
   const float rate = expf(a_log[head]), bias = dt_bias[head];
   // the batch's loads: lane l takes part (l % 4) of vector (l / 4): token (l / 8), q or k ((l / 4) % 2)
@@ -83,7 +112,7 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
 #pragma unroll
     for (int j = 0; j < VN; ++j) {
       const int idx = lane + j * WAVE, tt = idx / CW, pp = idx % CW;
-      vv[j] = (tt < nb && p0 + pp < P) ? load_as_float(qkv + (first + t0 + tt) * qkv_stride + v_col + head * P + p0 + pp) : 0.f;
+      vv[j] = (!unit && tt < nb && p0 + pp < P) ? load_as_float(qkv + (first + t0 + tt) * qkv_stride + v_col + head * P + p0 + pp) : 0.f;
     }
     if (lane < nb) {
       const float* gr = gates + (first + t0 + lane) * gate_stride;
@@ -145,6 +174,17 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
       }
       acc = lanes_sum<LPC>(acc);
       const float u = beta * (v - g * acc);
+      if (MODE == 1) {
+#pragma unroll
+        for (int i = 0; i < R4; ++i) {
+          if (i < rd4) {
+            const vf4 kk = kp[i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) S[4 * i + j] = g * S[4 * i + j] + kk[j] * u;
+          }
+        }
+        continue;
+      }
       float res = 0.f;
 #pragma unroll
       for (int i = 0; i < R4; ++i) {
@@ -161,12 +201,62 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
       if (sub == 0 && live) out[(first + t0 + tt) * (int64_t)(H * P) + head * P + p0 + col] = res;
     }
   }
-  if (write_state && live) {
+  if (MODE == 2 && seg != n_segs - 1) return;                     // the last segment leaves the sequence's state
+  float* to = MODE == 1 ? seg_mine : mine;
+  if ((MODE == 1 || write_state) && live) {
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
       const int d = sub * rd + i;
-      if (i < rd && d < D) mine[(int64_t)d * P] = S[i];
+      if (i < rd && d < D) to[unit ? d : (int64_t)d * P] = S[i];     // a column of A lies in one piece
     }
+  }
+}
+
+// The state that enters each segment of a sequence: S_in[0] is the sequence's own state, S_in[s + 1] =
+// A[s] S_in[s] + L[s]. One workgroup per (sequence, head, 8 columns), a thread a row of the state: the columns'
+// current values wait in LDS, every thread reads them all (broadcasts) against its row of A (`seg_trans` holds A
+// column by column, so that the threads of a wave read neighbouring words). `seg_state` holds L when the kernel
+// starts and S_in when it ends.
+#define DELTA_CARRY_COLS 8
+__global__ __launch_bounds__(DELTA_MAX_DIM) void delta_carry_kernel(
+    const int* __restrict__ seq_slot, const int* __restrict__ seg_cu, const float* __restrict__ state,
+    float* __restrict__ seg_state, const float* __restrict__ seg_trans, int H, int D, int P) {
+  __shared__ __attribute__((aligned(16))) float held[2][DELTA_MAX_DIM][DELTA_CARRY_COLS];
+  const int seq = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * DELTA_CARRY_COLS, d = threadIdx.x;
+  const int x0 = seg_cu[seq], n_segs = seg_cu[seq + 1] - x0, slot = seq_slot[seq];
+  if (slot < 0 || n_segs <= 0) return;
+  const bool row = d < D;
+  if (row) {
+    const float* src = state + (((int64_t)slot * H + head) * D + d) * P + p0;
+#pragma unroll
+    for (int c = 0; c < DELTA_CARRY_COLS; ++c) held[0][d][c] = p0 + c < P ? src[c] : 0.f;
+  }
+  __syncthreads();
+  int cur = 0;
+  for (int s = 0; s < n_segs; ++s) {
+    const bool last = s + 1 == n_segs;
+    if (row) {
+      float* at = seg_state + ((((int64_t)(x0 + s)) * H + head) * D + d) * P + p0;
+      float acc[DELTA_CARRY_COLS];
+#pragma unroll
+      for (int c = 0; c < DELTA_CARRY_COLS; ++c) {
+        acc[c] = (!last && p0 + c < P) ? at[c] : 0.f;
+        if (p0 + c < P) at[c] = held[cur][d][c];
+      }
+      if (!last) {
+        const float* a_row = seg_trans + (((int64_t)(x0 + s)) * H + head) * D * D + d;
+#pragma unroll 8
+        for (int e = 0; e < D; ++e) {
+          const float a = a_row[(int64_t)e * D];
+#pragma unroll
+          for (int c = 0; c < DELTA_CARRY_COLS; ++c) acc[c] += a * held[cur][e][c];
+        }
+#pragma unroll
+        for (int c = 0; c < DELTA_CARRY_COLS; ++c) held[cur ^ 1][d][c] = acc[c];
+      }
+    }
+    __syncthreads();
+    cur ^= 1;
   }
 }
 
@@ -189,25 +279,41 @@ DRYFT_API int dryft_delta_steps(const void* qkv, int64_t qkv_stride, int q_col, 
                                 int64_t gate_stride, int a_col, int b_col, const float* dt_bias, const float* a_log,
                                 const int* seq_slot, const int* cu_rows, const int* q_len, float* state, float* out,
                                 int n_seqs, int H, int G, int D, int P, float q_scale, float unit_eps, int write_state,
+                                const int* seg_cu, int max_segs, int seg_rows, float* seg_state, float* seg_trans,
                                 int is_f32, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || D > DELTA_MAX_DIM || P <= 0) return -1;
+  const bool cut = seg_cu != nullptr;
+  if (cut && (max_segs <= 0 || seg_rows <= 0 || seg_state == nullptr || seg_trans == nullptr || !write_state)) return -1;
+  const int walks = cut ? max_segs : n_seqs;
   // 16-byte loads of q and k: a lane's quarter of a vector in whole pieces of 8 values, at aligned addresses
   const int vec8 = (D % 32 == 0 && q_col % 8 == 0 && k_col % 8 == 0 && qkv_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0) ? 1 : 0;
-#define DELTA_LAUNCH(TT, L)                                                                                           \
-  hipLaunchKernelGGL((delta_steps_kernel<TT, L>), dim3(n_seqs, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0,   \
-                     stream, (const TT*)qkv, qkv_stride, q_col, k_col, v_col, gates, gate_stride, a_col, b_col, dt_bias, \
-                     a_log, seq_slot, cu_rows, q_len, state, out, H, G, D, P, q_scale, unit_eps, write_state, vec8)
-#define DELTA_PICK(TT)                                                                                                \
+  // MODE 1 walks the D columns of the unit matrix behind the P value columns
+#define DELTA_LAUNCH(TT, L, M)                                                                                        \
+  hipLaunchKernelGGL((delta_steps_kernel<TT, L, M>),                                                                  \
+                     dim3(walks, H, (P + WAVE / L - 1) / (WAVE / L) + (M == 1 ? (D + WAVE / L - 1) / (WAVE / L) : 0)), \
+                     dim3(WAVE), 0, stream, (const TT*)qkv, qkv_stride, q_col, k_col, v_col, gates, gate_stride, a_col, \
+                     b_col, dt_bias, a_log, seq_slot, cu_rows, q_len, state, out, H, G, D, P, q_scale, unit_eps,      \
+                     write_state, vec8, seg_cu, n_seqs, seg_rows, seg_state, seg_trans)
+#define DELTA_PICK(TT, M)                                                                                             \
   switch (lpc) {                                                                                                      \
-    case 16: DELTA_LAUNCH(TT, 16); break;                                                                             \
-    case 8: DELTA_LAUNCH(TT, 8); break;                                                                               \
-    case 4: DELTA_LAUNCH(TT, 4); break;                                                                               \
-    case 2: DELTA_LAUNCH(TT, 2); break;                                                                               \
-    default: DELTA_LAUNCH(TT, 1);                                                                                     \
+    case 16: DELTA_LAUNCH(TT, 16, M); break;                                                                          \
+    case 8: DELTA_LAUNCH(TT, 8, M); break;                                                                            \
+    case 4: DELTA_LAUNCH(TT, 4, M); break;                                                                            \
+    case 2: DELTA_LAUNCH(TT, 2, M); break;                                                                            \
+    default: DELTA_LAUNCH(TT, 1, M);                                                                                  \
   }
-  const int lpc = lanes_per_column(D, n_seqs, H, P);
-  if (is_f32) { DELTA_PICK(float) } else { DELTA_PICK(bf16_t) }
+#define DELTA_RUN(M) if (is_f32) { DELTA_PICK(float, M) } else { DELTA_PICK(bf16_t, M) }
+  const int lpc = lanes_per_column(D, walks, H, P);
+  if (!cut) {
+    DELTA_RUN(0)
+  } else {
+    DELTA_RUN(1)
+    hipLaunchKernelGGL(delta_carry_kernel, dim3(n_seqs, H, (P + DELTA_CARRY_COLS - 1) / DELTA_CARRY_COLS),
+                       dim3((D + WAVE - 1) / WAVE * WAVE), 0, stream, seq_slot, seg_cu, state, seg_state, seg_trans, H, D, P);
+    DELTA_RUN(2)
+  }
+#undef DELTA_RUN
 #undef DELTA_PICK
 #undef DELTA_LAUNCH
   return DRYFT_LAUNCH_CHECK();

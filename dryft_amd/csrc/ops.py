@@ -95,11 +95,12 @@ _SIGNATURES = {
              "dryft_causal_conv": [_P, _L, _I, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
              "dryft_conv_tail": [_P, _L, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P]},
     "ssm": {"dryft_ssm_max_state": [],
-            "dryft_ssm_scan": [_P, _L, _I, _I, _I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+            "dryft_ssm_scan": [_P, _L, _I, _I, _I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I,
+                               _I, _P, _P, _I, _P],
             "dryft_gate_part_norm": [_P, _P, _L, _I, _P, _P, _P, _I, _I, _I, _F, _I, _P]},
     "delta": {"dryft_delta_max_dim": [],
               "dryft_delta_steps": [_P, _L, _I, _I, _I, _P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I,
-                                    _F, _F, _I, _I, _P]},
+                                    _F, _F, _I, _P, _I, _I, _P, _P, _I, _P]},
     "sampling": {"dryft_argmax_rows": [_P, _I, _I, _L, _P, _I, _P, _P, _P],
                  "dryft_sample_rows": [_P, _I, _I, _L, _F, _P, _P, _I, _P, _P, _P]},
 }
@@ -1856,13 +1857,28 @@ def norm_rope_half_kv(src, q_col: int, k_col: int, v_col: int, q_weight, k_weigh
 SSM_MAX_STATE = 256
 
 
+def _segment_facts(who: str, segments, n_seqs: int, write_state: bool):
+    """``(rows per segment, prefix sums, bound)`` of a walk cut into segments, checked; zeros and None for a whole walk."""
+    if segments is None:
+        return 0, None, 0
+    seg_rows, seg_cu, max_segs = segments
+    _gpu(seg_cu, "segment prefix sums", torch.int32)
+    if not (seg_cu.numel() >= n_seqs + 1 and seg_rows > 0 and write_state):
+        raise KernelError(f"{who}: segments of a positive number of rows, prefix sums for every sequence, and a state "
+                          "that is written back")
+    return int(seg_rows), seg_cu, int(max_segs)
+
+
 def ssm_scan(xbc, x_col: int, b_col: int, c_col: int, dt_raw, dt_bias, a_log, d_skip, seq_slot, cu_rows, q_len,
-             n_seqs: int, state, y, n_heads: int, head_dim: int, n_state: int, groups: int, write_state: bool) -> None:
+             n_seqs: int, state, y, n_heads: int, head_dim: int, n_state: int, groups: int, write_state: bool,
+             segments=None) -> None:
     """Per sequence and head, over the sequence's rows of the step in order, from ``state [slots, heads, n_state,
     head_dim]`` (float32): ``dt = softplus(dt_raw + dt_bias)``, ``S <- exp(-exp(a_log) dt) S + dt B x^T``,
     ``y = S^T C + d_skip x``. ``x [heads, head_dim]``, ``B`` and ``C [groups, n_state]`` are runs of columns of ``xbc``
     (activation dtype), ``dt_raw`` float32 ``[rows, >= heads]``, ``y`` float32 ``[rows, heads * head_dim]`` (rows of
-    sequences that sit out are not written)."""
+    sequences that sit out are not written). ``segments = (rows per segment, prefix sums of segments over the
+    sequences, their bound)``: long sequences run as segments side by side, in three launches (every segment's summary
+    from a zero state, the state that enters each, every segment's read-outs)."""
     _gpu(xbc, "xbc")
     rows = xbc.shape[0]
     inner = n_heads * head_dim
@@ -1883,10 +1899,18 @@ def ssm_scan(xbc, x_col: int, b_col: int, c_col: int, dt_raw, dt_bias, a_log, d_
         raise KernelError("ssm_scan: y must be contiguous float32 [rows, heads * head_dim]")
     if not (0 < n_state <= SSM_MAX_STATE and groups > 0 and n_heads % groups == 0):
         raise KernelError(f"ssm_scan: a state of 1..{SSM_MAX_STATE} rows, heads a multiple of groups")
+    seg_rows, seg_cu, max_segs = _segment_facts("ssm_scan", segments, n_seqs, write_state)
+    if segments is not None and max_segs <= 0:
+        return
+    seg_state = seg_decay = None
+    if segments is not None:
+        seg_state = torch.empty((max_segs, n_heads, n_state, head_dim), dtype=torch.float32, device=xbc.device)
+        seg_decay = torch.empty((max_segs, n_heads), dtype=torch.float32, device=xbc.device)
     _check(_fn("ssm", "dryft_ssm_scan")(_ptr(xbc), xbc.stride(0), x_col, b_col, c_col, _ptr(dt_raw), dt_raw.stride(0),
                                         _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(seq_slot), _ptr(cu_rows),
                                         _ptr(q_len), _ptr(state), _ptr(y), n_seqs, n_heads, head_dim, n_state, groups,
-                                        int(bool(write_state)), _float_flag(xbc, "xbc"), _stream()), "ssm_scan")
+                                        int(bool(write_state)), _ptr(seg_cu), max_segs, seg_rows, _ptr(seg_state),
+                                        _ptr(seg_decay), _float_flag(xbc, "xbc"), _stream()), "ssm_scan")
 
 
 def gate_part_norm(y, z, z_col: int, weight, row_slot, out, parts: int, eps: float) -> None:
@@ -1914,12 +1938,15 @@ DELTA_MAX_DIM = 256
 
 def delta_steps(qkv, q_col: int, k_col: int, v_col: int, gates, a_col: int, b_col: int, dt_bias, a_log, seq_slot, cu_rows,
                 q_len, n_seqs: int, state, out, n_heads: int, n_groups: int, key_dim: int, value_dim: int, q_scale: float,
-                unit_eps: float, write_state: bool) -> None:
+                unit_eps: float, write_state: bool, segments=None) -> None:
     """Per sequence and head, over the sequence's rows of the step in order, from ``state [slots, heads, key_dim,
     value_dim]`` (float32): ``S <- g S``, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q`` with
     ``g = exp(-exp(a_log) softplus(gates[:, a_col + h] + dt_bias))``, ``beta = sigmoid(gates[:, b_col + h])``, q and k
     (``n_groups`` of them, runs of columns of ``qkv``) made unit vectors with ``unit_eps`` under the root, q times
-    ``q_scale``. ``out`` float32 ``[rows, heads * value_dim]`` (rows of sequences that sit out are not written)."""
+    ``q_scale``. ``out`` float32 ``[rows, heads * value_dim]`` (rows of sequences that sit out are not written).
+    ``segments = (rows per segment, prefix sums of segments over the sequences, their bound)``: long sequences run as
+    segments side by side, in three launches (every segment's summary, the state it reaches from zero and the map it
+    applies to the state that enters it; the state that enters each; every segment's read-outs)."""
     _gpu(qkv, "qkv")
     rows = qkv.shape[0]
     if not (qkv.dim() == 2 and qkv.stride(1) == 1 and min(q_col, k_col, v_col) >= 0 and
@@ -1940,8 +1967,15 @@ def delta_steps(qkv, q_col: int, k_col: int, v_col: int, gates, a_col: int, b_co
         raise KernelError("delta_steps: out must be contiguous float32 [rows, heads * value_dim]")
     if not (0 < key_dim <= DELTA_MAX_DIM and n_groups > 0 and n_heads % n_groups == 0):
         raise KernelError(f"delta_steps: keys of 1..{DELTA_MAX_DIM} features, heads a multiple of the key heads")
+    seg_rows, seg_cu, max_segs = _segment_facts("delta_steps", segments, n_seqs, write_state)
+    if segments is not None and max_segs <= 0:
+        return
+    seg_state = seg_trans = None
+    if segments is not None:
+        seg_state = torch.empty((max_segs, n_heads, key_dim, value_dim), dtype=torch.float32, device=qkv.device)
+        seg_trans = torch.empty((max_segs, n_heads, key_dim, key_dim), dtype=torch.float32, device=qkv.device)
     _check(_fn("delta", "dryft_delta_steps")(
         _ptr(qkv), qkv.stride(0), q_col, k_col, v_col, _ptr(gates), gates.stride(0), a_col, b_col, _ptr(dt_bias),
         _ptr(a_log), _ptr(seq_slot), _ptr(cu_rows), _ptr(q_len), _ptr(state), _ptr(out), n_seqs, n_heads, n_groups,
-        key_dim, value_dim, float(q_scale), float(unit_eps), int(bool(write_state)), _float_flag(qkv, "qkv"), _stream()),
-        "delta_steps")
+        key_dim, value_dim, float(q_scale), float(unit_eps), int(bool(write_state)), _ptr(seg_cu), max_segs, seg_rows,
+        _ptr(seg_state), _ptr(seg_trans), _float_flag(qkv, "qkv"), _stream()), "delta_steps")

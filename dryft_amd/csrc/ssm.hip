@@ -21,12 +21,22 @@
 
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-template <typename T, int LPC>
+//
+// Long prompts are cut into segments of `seg_rows` rows that run side by side (MODE 1, then the carry kernel, then
+// MODE 2; MODE 0 walks a whole sequence). The recurrence is linear in the state and its decay one number per head
+// and token, so a segment's effect is S_out = p S_in + L with p the product of the segment's decays and L the state
+// it reaches from zero. MODE 1 computes L and p of every segment but a sequence's last (no read-outs); the carry
+// kernel walks a sequence's segments and leaves each the state that enters it; MODE 2 starts every segment from that
+// state and writes its read-outs, and a sequence's last segment writes the state back. Segment x of the step belongs
+// to the sequence s with seg_cu[s] <= x < seg_cu[s + 1] (prefix sums over the sequences; one that sits out has none).
+template <typename T, int LPC, int MODE>
 __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     const T* __restrict__ xbc, int64_t xbc_stride, int x_col, int b_col, int c_col, const float* __restrict__ dt_raw,
     int64_t dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
     const int* __restrict__ seq_slot, const int* __restrict__ cu_rows, const int* __restrict__ q_len,
-    float* __restrict__ state, float* __restrict__ y, int H, int P, int N, int G, int write_state, int vec8) {
+    float* __restrict__ state, float* __restrict__ y, int H, int P, int N, int G, int write_state, int vec8,
+    const int* __restrict__ seg_cu, int n_seqs, int seg_rows, float* __restrict__ seg_state,
+    float* __restrict__ seg_decay) {
   constexpr int CW = WAVE / LPC;                       // columns a wave owns
   constexpr int ROWS = SSM_MAX_STATE / LPC < SSM_ROWS ? SSM_MAX_STATE / LPC : SSM_ROWS;
   constexpr int R4 = ROWS / 4;
@@ -37,21 +47,34 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
   __shared__ __attribute__((aligned(16))) float sB[SSM_BATCH][SSM_MAX_STATE + 8 * LPC];
   __shared__ __attribute__((aligned(16))) float sC[SSM_BATCH][SSM_MAX_STATE + 8 * LPC];
   __shared__ float sx[SSM_BATCH][CW], sdt[SSM_BATCH], sa[SSM_BATCH];
-  const int seq = blockIdx.x, head = blockIdx.y, p0 = blockIdx.z * CW;
-  const int slot = seq_slot[seq], rows = q_len[seq];
+  const int head = blockIdx.y, p0 = blockIdx.z * CW;
+  int seq = blockIdx.x, seg = 0, n_segs = 1;
+  if (MODE != 0) {
+    if ((int)blockIdx.x >= seg_cu[n_seqs]) return;
+    seq = 0;
+    while (seg_cu[seq + 1] <= (int)blockIdx.x) ++seq;
+    seg = blockIdx.x - seg_cu[seq];
+    n_segs = seg_cu[seq + 1] - seg_cu[seq];
+    if (MODE == 1 && seg == n_segs - 1) return;                   // nobody needs the last segment's summary
+  }
+  const int slot = seq_slot[seq];
+  const int rows = MODE == 0 ? q_len[seq] : min(seg_rows, q_len[seq] - seg * seg_rows);
   if (slot < 0 || rows <= 0) return;
-  const int64_t first = cu_rows[seq];
+  const int64_t first = cu_rows[seq] + (MODE == 0 ? 0 : seg * seg_rows);
   const int group = head / (H / G);
   const int lane = threadIdx.x, sub = lane % LPC, col = lane / LPC;
   const bool live = p0 + col < P;
   const int rd = (N + LPC - 1) / LPC, rd4 = (rd + 3) / 4, run = 4 * rd4 + 4;
   float* mine = state + (((int64_t)slot * H + head) * N) * P + p0 + col;
+  float* seg_mine = MODE == 0 ? nullptr : seg_state + (((int64_t)blockIdx.x * H + head) * N) * P + p0 + col;
+  const float* from = MODE == 2 ? seg_mine : mine;
   float S[ROWS];
 #pragma unroll
   for (int i = 0; i < ROWS; ++i) {
     const int n = sub * rd + i;
-    S[i] = (live && i < rd && n < N) ? mine[(int64_t)n * P] : 0.f;
+    S[i] = (MODE != 1 && live && i < rd && n < N) ? from[(int64_t)n * P] : 0.f;
   }
+  float decays = 1.f;
   const float rate = expf(a_log[head]), bias = dt_bias[head], skip = d_skip[head];
   // the batch's loads: lane l takes part (l % 4) of vector (l / 4): token (l / 8), B or C ((l / 4) % 2)
   const int vec = lane / 4, part = lane % 4, v_tok = vec >> 1, v_is_c = vec & 1;
@@ -121,6 +144,18 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     for (int tt = 0; tt < nb; ++tt) {
       const float a = sa[tt], x = sx[tt][col], dtx = sdt[tt] * x;
       const vf4* bp = (const vf4*)(sB[tt] + sub * run);
+      if (MODE == 1) {
+        decays *= a;
+#pragma unroll
+        for (int i = 0; i < R4; ++i) {
+          if (i < rd4) {
+            const vf4 bb = bp[i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) S[4 * i + j] = a * S[4 * i + j] + dtx * bb[j];
+          }
+        }
+        continue;
+      }
       const vf4* cp = (const vf4*)(sC[tt] + sub * run);
       float acc = 0.f;
 #pragma unroll
@@ -138,12 +173,32 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
       if (sub == 0 && live) y[(first + t0 + tt) * (int64_t)(H * P) + head * P + p0 + col] = acc + skip * x;
     }
   }
-  if (write_state && live) {
+  if (MODE == 1 && blockIdx.z == 0 && lane == 0) seg_decay[(int64_t)blockIdx.x * H + head] = decays;
+  if (MODE == 2 && seg != n_segs - 1) return;                     // the last segment leaves the sequence's state
+  float* to = MODE == 1 ? seg_mine : mine;
+  if ((MODE == 1 || write_state) && live) {
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
       const int n = sub * rd + i;
-      if (i < rd && n < N) mine[(int64_t)n * P] = S[i];
+      if (i < rd && n < N) to[(int64_t)n * P] = S[i];
     }
+  }
+}
+
+// The state that enters each segment of a sequence: S_in[0] is the sequence's own state, S_in[s + 1] =
+// p[s] S_in[s] + L[s]. A thread an entry of the state; `seg_state` holds L when the kernel starts and S_in when it ends.
+__global__ __launch_bounds__(256) void ssm_carry_kernel(const int* __restrict__ seq_slot, const int* __restrict__ seg_cu,
+                                                        const float* __restrict__ state, float* __restrict__ seg_state,
+                                                        const float* __restrict__ seg_decay, int H, int entries) {
+  const int seq = blockIdx.x, head = blockIdx.y, e = blockIdx.z * 256 + threadIdx.x;
+  const int x0 = seg_cu[seq], n_segs = seg_cu[seq + 1] - x0, slot = seq_slot[seq];
+  if (slot < 0 || e >= entries) return;
+  float held = state[((int64_t)slot * H + head) * entries + e];
+  for (int s = 0; s < n_segs; ++s) {
+    float* at = seg_state + ((int64_t)(x0 + s) * H + head) * entries + e;
+    const float local = s + 1 < n_segs ? *at : 0.f;
+    *at = held;
+    if (s + 1 < n_segs) held = seg_decay[(int64_t)(x0 + s) * H + head] * held + local;
   }
 }
 
@@ -195,25 +250,39 @@ static int lanes_per_column(int rows_of_state, int n_seqs, int heads, int column
 DRYFT_API int dryft_ssm_scan(const void* xbc, int64_t xbc_stride, int x_col, int b_col, int c_col, const float* dt_raw,
                              int64_t dt_stride, const float* dt_bias, const float* a_log, const float* d_skip,
                              const int* seq_slot, const int* cu_rows, const int* q_len, float* state, float* y, int n_seqs,
-                             int H, int P, int N, int G, int write_state, int is_f32, hipStream_t stream) {
+                             int H, int P, int N, int G, int write_state, const int* seg_cu, int max_segs, int seg_rows,
+                             float* seg_state, float* seg_decay, int is_f32, hipStream_t stream) {
   if (n_seqs <= 0) return 0;
   if (H <= 0 || P <= 0 || N <= 0 || N > SSM_MAX_STATE || G <= 0 || H % G) return -1;
+  const bool cut = seg_cu != nullptr;
+  if (cut && (max_segs <= 0 || seg_rows <= 0 || seg_state == nullptr || seg_decay == nullptr || !write_state)) return -1;
+  const int walks = cut ? max_segs : n_seqs;
   // 16-byte loads of B and C: a lane's quarter of a vector in whole pieces of 8 values, at aligned addresses
   const int vec8 = (N % 32 == 0 && b_col % 8 == 0 && c_col % 8 == 0 && xbc_stride % 8 == 0 && ((uintptr_t)xbc & 15) == 0) ? 1 : 0;
-#define SSM_LAUNCH(TT, L)                                                                                             \
-  hipLaunchKernelGGL((ssm_scan_kernel<TT, L>), dim3(n_seqs, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0, stream, \
+#define SSM_LAUNCH(TT, L, M)                                                                                          \
+  hipLaunchKernelGGL((ssm_scan_kernel<TT, L, M>), dim3(walks, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0, stream, \
                      (const TT*)xbc, xbc_stride, x_col, b_col, c_col, dt_raw, dt_stride, dt_bias, a_log, d_skip,      \
-                     seq_slot, cu_rows, q_len, state, y, H, P, N, G, write_state, vec8)
-#define SSM_PICK(TT)                                                                                                  \
+                     seq_slot, cu_rows, q_len, state, y, H, P, N, G, write_state, vec8, seg_cu, n_seqs, seg_rows,     \
+                     seg_state, seg_decay)
+#define SSM_PICK(TT, M)                                                                                               \
   switch (lpc) {                                                                                                      \
-    case 16: SSM_LAUNCH(TT, 16); break;                                                                               \
-    case 8: SSM_LAUNCH(TT, 8); break;                                                                                 \
-    case 4: SSM_LAUNCH(TT, 4); break;                                                                                 \
-    case 2: SSM_LAUNCH(TT, 2); break;                                                                                 \
-    default: SSM_LAUNCH(TT, 1);                                                                                       \
+    case 16: SSM_LAUNCH(TT, 16, M); break;                                                                            \
+    case 8: SSM_LAUNCH(TT, 8, M); break;                                                                              \
+    case 4: SSM_LAUNCH(TT, 4, M); break;                                                                              \
+    case 2: SSM_LAUNCH(TT, 2, M); break;                                                                              \
+    default: SSM_LAUNCH(TT, 1, M);                                                                                    \
   }
-  const int lpc = lanes_per_column(N, n_seqs, H, P);
-  if (is_f32) { SSM_PICK(float) } else { SSM_PICK(bf16_t) }
+#define SSM_RUN(M) if (is_f32) { SSM_PICK(float, M) } else { SSM_PICK(bf16_t, M) }
+  const int lpc = lanes_per_column(N, walks, H, P);
+  if (!cut) {
+    SSM_RUN(0)
+  } else {
+    SSM_RUN(1)
+    hipLaunchKernelGGL(ssm_carry_kernel, dim3(n_seqs, H, (N * P + 255) / 256), dim3(256), 0, stream, seq_slot, seg_cu,
+                       state, seg_state, seg_decay, H, N * P);
+    SSM_RUN(2)
+  }
+#undef SSM_RUN
 #undef SSM_PICK
 #undef SSM_LAUNCH
   return DRYFT_LAUNCH_CHECK();

@@ -79,6 +79,18 @@ class StepContext:
             found = self._tiles[rows_per_tile] = (tile_cu, bound)
         return found
 
+    def segments(self, multiple: int = 1, shortest: int = 64, most: int = 16):
+        """How a walk over the step's long sequences is cut so that the pieces run side by side: ``(rows per segment,
+        prefix sums of segments over the sequences, their bound)``, with segments of at least ``shortest`` rows in
+        multiples of ``multiple`` and at most ``most`` for the longest sequence (every segment but a sequence's last
+        is walked more than once, so short sequences stay whole); None for steps whose sequences are all short."""
+        if self.max_q_len < 2 * shortest:
+            return None
+        per = -(-self.max_q_len // most)
+        seg_rows = max(shortest, -(-per // multiple) * multiple)
+        seg_cu, bound = self.tiles(seg_rows)
+        return seg_rows, seg_cu, bound
+
     def kept_zeros(self, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         """A tensor that starts as zeros and lives as long as the context, one per shape and dtype, shared by every
         part that asks: for an output of which a kernel writes only the rows of sequences that take part, while the

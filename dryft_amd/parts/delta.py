@@ -12,7 +12,9 @@ a weight shared by the heads, times ``silu(W_g h)``, and projected back.
 
 The state (``S`` and the convolution's last ``taps - 1`` inputs) is float32 in the state store, zero when a sequence
 starts. The two gates keep the float32 accumulators of their projections; sigmoid, softplus, both exponentials, the
-unit lengths, the recurrence and the read-out's norm are float arithmetic in both precisions.
+unit lengths, the recurrence and the read-out's norm are float arithmetic in both precisions. A long sequence of a step
+is walked as segments side by side: a token maps every column of the state alike, ``c -> g (I - beta k k^T) c + beta k
+v_c``, so a segment's effect is the product of its tokens' maps and the state it reaches from zero.
 """
 
 from __future__ import annotations
@@ -80,9 +82,12 @@ class GatedDeltaMixer(Mixer):
         # the rows of sequences that sit out are not visited by the walk; the read-out norms whatever they hold
         o_raw = ctx.kept_zeros((rows, self.v_dim), torch.float32) if ctx.some_sit_out() else \
             torch.empty((rows, self.v_dim), dtype=torch.float32, device=h.device)
+        # a long prompt runs as segments side by side
+        segments = ctx.segments() if writes_cache else None
         ops.delta_steps(qkv, 0, self.qk_dim, 2 * self.qk_dim, gates, 0, self.n_heads, self.dt_bias, self.a_log,
                         ctx.seq_slot, ctx.cu_rows, ctx.q_len, ctx.n_seqs, line["memory"].state, o_raw, self.n_heads,
-                        self.n_kv, self.key_dim, self.value_dim, self.key_dim ** -0.5, self.unit_eps, writes_cache)
+                        self.n_kv, self.key_dim, self.value_dim, self.key_dim ** -0.5, self.unit_eps, writes_cache,
+                        segments=segments)
         out = torch.empty((rows, self.v_dim), dtype=h.dtype, device=h.device)
         ops.wkv_out(o_raw, proj[:, self.conv_channels:], self.out_norm, out, self.n_heads, self.value_dim, self.norm_eps)
         return linear(out, self.w_o, allow_partials=True)

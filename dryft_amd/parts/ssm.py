@@ -13,7 +13,9 @@ projected back.
 The state (``S`` and the convolution's last ``taps - 1`` inputs) is float32 in the state store, zero when a sequence
 starts. The step sizes keep the float32 accumulators of their projection, and softplus, both exponentials, the
 recurrence, the gate and the norm are float arithmetic in both precisions. A step may bring any number of rows per
-sequence; the kernels walk them in order from the state the step before left.
+sequence; the kernels walk them in order from the state the step before left, a long sequence as segments side by side
+(the recurrence is linear in the state: a segment's effect is the product of its decays and the state it reaches from
+zero).
 """
 
 from __future__ import annotations
@@ -80,10 +82,12 @@ class StateSpaceMixer(Mixer):
         dt_raw = linear(h, self.w_dt, out_dtype=torch.float32)
         xbc = short_conv(proj, self.inner, self.conv_channels, self.conv_w, ctx, line.get("tail"), writes_cache,
                          out_bias=self.conv_b, silu=True)
+        # a long prompt runs as segments side by side (the rows of sequences that sit out are then not visited)
+        segments = ctx.segments() if writes_cache else None
         y = torch.empty((rows, self.inner), dtype=torch.float32, device=h.device)
         ops.ssm_scan(xbc, 0, self.inner, self.inner + GN, dt_raw, self.dt_bias, self.a_log, self.d_skip, ctx.seq_slot,
                      ctx.cu_rows, ctx.q_len, ctx.n_seqs, line["state"].state, y, self.n_heads, self.head_dim,
-                     self.n_state, self.groups, writes_cache)
+                     self.n_state, self.groups, writes_cache, segments=segments)
         out = torch.empty((rows, self.inner), dtype=h.dtype, device=h.device)
         ops.gate_part_norm(y, proj, 0, self.out_norm, ctx.row_slot, out, self.norm_parts, self.norm_eps)
         return linear(out, self.w_o, allow_partials=True)

@@ -25,8 +25,6 @@ from .base import Mixer, StepContext, matrix
 from .linear import linear
 
 _BLENDS = ("r", "k", "v", "g", "w")
-_SEGMENT_ROWS = 64       # the shortest segment a long sequence is cut into
-_MAX_SEGMENTS = 16       # the most segments of one sequence
 
 
 class WKVMixer(Mixer):
@@ -77,7 +75,7 @@ class WKVMixer(Mixer):
         decay = torch.empty((rows, self.inner), dtype=torch.float32, device=h.device)
         ops.wkv_decay(low, self.w_up, self.decay_bias, decay)
         # a long prompt runs as segments side by side (the rows of sequences that sit out are then not visited)
-        segments = self._segments(ctx) if writes_cache else None
+        segments = ctx.segments(ops.WKV_GROUP) if writes_cache else None
         if segments is not None and ctx.some_sit_out():
             o_raw = ctx.kept_zeros((rows, self.inner), torch.float32)
         else:
@@ -88,18 +86,6 @@ class WKVMixer(Mixer):
         out = torch.empty((rows, self.inner), dtype=h.dtype, device=h.device)
         ops.wkv_out(o_raw, g, self.out_norm, out, self.n_heads, self.head_dim, self.norm_eps)
         return linear(out, self.w_o, allow_partials=True)
-
-    @staticmethod
-    def _segments(ctx: StepContext):
-        """How a step's long sequences are cut: segments of at least ``_SEGMENT_ROWS`` rows, at most ``_MAX_SEGMENTS``
-        for the longest sequence (every segment but a sequence's last is walked twice, so short sequences stay
-        whole); None for steps whose sequences are all short."""
-        if ctx.max_q_len < 2 * _SEGMENT_ROWS:
-            return None
-        per = -(-ctx.max_q_len // _MAX_SEGMENTS)
-        seg_rows = max(_SEGMENT_ROWS, -(-per // ops.WKV_GROUP) * ops.WKV_GROUP)
-        seg_cu, bound = ctx.tiles(seg_rows)
-        return seg_rows, seg_cu, bound
 
     def flops(self, rows, spans):
         """The projections, and per token and head the update of the state and its read-out."""

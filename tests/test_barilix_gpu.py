@@ -317,6 +317,31 @@ def test_delta_rule_keeps_an_early_token_and_reads_its_own_write(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["state-space", "delta-odd", "delta-real"])
+def test_long_prompts_walked_as_segments(dtype, kind):
+    """Long sequences of a step are cut into segments that run side by side and are joined through each segment's
+    summary: sequences that fill a whole number of segments, one row more, many segments, and too few rows to be cut,
+    in one step; then the same from a state that an earlier step left, and with a last portion of one row."""
+    if kind == "state-space":
+        m = state_space(4, 16, 24, 2, 3, 2)
+        cfg, t, plan = mixer_case(parallel(attention(1, 1, 8, 8, 1), m), 48, seed=3)
+        part, cache, positions = load_mixer(plan, t, dtype, max_len=512, branch="right")
+        w = sub(t, "l0.mix.right.")
+        plain = lambda s: P.state_space(s.double(), w, m, EPS)[0]
+    else:
+        layer = delta(2, 1, 40, 72, 2) if kind == "delta-odd" else delta(2, 2, 128, 128, 4)
+        cfg, t, plan = mixer_case(layer, 48, seed=4)
+        part, cache, positions = load_mixer(plan, t, dtype, max_len=512)
+        w = sub(t, "l0.mix.")
+        plain = lambda s: P.delta_mixer(s.double(), w, layer["mixer"], EPS)[0]
+    seqs = inputs(dtype, 48, lengths=(450, 128, 129, 30), seed=21)
+    want = [plain(s) for s in seqs]
+    for cuts in ([], [150], [129, 449]):
+        for got, ref in zip(run_mixer(part, cache, positions, dtype, seqs, cuts), want):
+            assert rel_err(got, ref) <= MIXER_TOL[dtype], (kind, cuts)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_parallel_mixers_alone(dtype):
     layer = CASES["A"]["layers"][1]
     layer = parallel(layer["mixer"]["left"], layer["mixer"]["right"])
