@@ -35,7 +35,7 @@ __device__ __forceinline__ float softplus_d(float z) { return z > 20.f ? z : log
 // the state that enters it; MODE 2 starts every segment from that state and writes its read-outs, and a sequence's
 // last segment writes the state back. Segment x of the step belongs to the sequence s with seg_cu[s] <= x <
 // seg_cu[s + 1] (prefix sums over the sequences; one that sits out has none).
-template <typename T, int LPC, int MODE>
+template <typename T, int LPC, int MODE, int MAXN>
 __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
     const T* __restrict__ qkv, int64_t qkv_stride, int q_col, int k_col, int v_col, const float* __restrict__ gates,
     int64_t gate_stride, int a_col, int b_col, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
@@ -44,14 +44,14 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
     int write_state, int vec8, const int* __restrict__ seg_cu, int n_seqs, int seg_rows, float* __restrict__ seg_state,
     float* __restrict__ seg_trans) {
   constexpr int CW = WAVE / LPC;                       // columns a wave owns
-  constexpr int ROWS = DELTA_MAX_DIM / LPC < DELTA_ROWS ? DELTA_MAX_DIM / LPC : DELTA_ROWS;
+  constexpr int ROWS = MAXN / LPC < DELTA_ROWS ? MAXN / LPC : DELTA_ROWS;
   constexpr int R4 = ROWS / 4;
-  constexpr int PER = DELTA_MAX_DIM / 4;               // values of a q or k vector one of its four lanes takes at most
+  constexpr int PER = MAXN / 4;                // values of a q or k vector one of its four lanes takes at most
   constexpr int VN = (DELTA_BATCH * CW + WAVE - 1) / WAVE;
   // a vector in LDS: LPC runs (the rows of one lane each), a run padded with zeros to a multiple of 4 floats and
   // followed by 4 more so that neighbouring runs start in different banks
-  __shared__ __attribute__((aligned(16))) float sk[DELTA_BATCH][DELTA_MAX_DIM + 8 * LPC];
-  __shared__ __attribute__((aligned(16))) float sq[DELTA_BATCH][DELTA_MAX_DIM + 8 * LPC];
+  __shared__ __attribute__((aligned(16))) float sk[DELTA_BATCH][MAXN + 8 * LPC];
+  __shared__ __attribute__((aligned(16))) float sq[DELTA_BATCH][MAXN + 8 * LPC];
   __shared__ float sv[DELTA_BATCH][CW], sg[DELTA_BATCH], sbeta[DELTA_BATCH];
   const int head = blockIdx.y, z_values = (P + CW - 1) / CW;
   const bool unit = MODE == 1 && (int)blockIdx.z >= z_values;      // this wave walks columns of the unit matrix
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
     }
   };
   if (4 * rd4 != rd || rd * LPC != D) {                // what pads the runs stays zero for good
-    for (int i = lane; i < DELTA_BATCH * (DELTA_MAX_DIM + 8 * LPC); i += WAVE) { (&sk[0][0])[i] = 0.f; (&sq[0][0])[i] = 0.f; }
+    for (int i = lane; i < DELTA_BATCH * (MAXN + 8 * LPC); i += WAVE) { (&sk[0][0])[i] = 0.f; (&sq[0][0])[i] = 0.f; }
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
@@ -263,13 +263,13 @@ __global__ __launch_bounds__(DELTA_MAX_DIM) void delta_carry_kernel(
 DRYFT_API int dryft_delta_max_dim() { return DELTA_MAX_DIM; }
 
 // Lanes a column: as few as hold its rows (64 each), then more while every lane keeps eight rows or more and the
-// launch stays within a wave per SIMD of the chip.
-static int lanes_per_column(int rows_of_state, int n_seqs, int heads, int columns) {
+// launch stays within `most` waves.
+static int lanes_per_column(int rows_of_state, int walks, int heads, int columns, int most) {
   int lpc = rows_of_state > 128 ? 4 : (rows_of_state > 64 ? 2 : 1);
   while (lpc < 16) {
     const int next = 2 * lpc, cw = WAVE / next;
     if ((rows_of_state + next - 1) / next < 8) break;
-    if ((int64_t)n_seqs * heads * ((columns + cw - 1) / cw) > 1024 && cw < columns) break;
+    if ((int64_t)walks * heads * ((columns + cw - 1) / cw) > most && cw < columns) break;
     lpc = next;
   }
   return lpc;
@@ -288,23 +288,26 @@ DRYFT_API int dryft_delta_steps(const void* qkv, int64_t qkv_stride, int q_col, 
   const int walks = cut ? max_segs : n_seqs;
   // 16-byte loads of q and k: a lane's quarter of a vector in whole pieces of 8 values, at aligned addresses
   const int vec8 = (D % 32 == 0 && q_col % 8 == 0 && k_col % 8 == 0 && qkv_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0) ? 1 : 0;
-  // MODE 1 walks the D columns of the unit matrix behind the P value columns
-#define DELTA_LAUNCH(TT, L, M)                                                                                        \
-  hipLaunchKernelGGL((delta_steps_kernel<TT, L, M>),                                                                  \
+  // MODE 1 walks the D columns of the unit matrix behind the P value columns. The kernel is built for states of up
+  // to 64, 128 and 256 rows (X), so that a lane's registers and the loops over them fit the state at hand.
+#define DELTA_LAUNCH(TT, L, M, X)                                                                                     \
+  hipLaunchKernelGGL((delta_steps_kernel<TT, L, M, X>),                                                               \
                      dim3(walks, H, (P + WAVE / L - 1) / (WAVE / L) + (M == 1 ? (D + WAVE / L - 1) / (WAVE / L) : 0)), \
                      dim3(WAVE), 0, stream, (const TT*)qkv, qkv_stride, q_col, k_col, v_col, gates, gate_stride, a_col, \
                      b_col, dt_bias, a_log, seq_slot, cu_rows, q_len, state, out, H, G, D, P, q_scale, unit_eps,      \
                      write_state, vec8, seg_cu, n_seqs, seg_rows, seg_state, seg_trans)
+#define DELTA_CASE(TT, M, X, L) if (maxn == X && lpc == L) { DELTA_LAUNCH(TT, L, M, X); } else
 #define DELTA_PICK(TT, M)                                                                                             \
-  switch (lpc) {                                                                                                      \
-    case 16: DELTA_LAUNCH(TT, 16, M); break;                                                                          \
-    case 8: DELTA_LAUNCH(TT, 8, M); break;                                                                            \
-    case 4: DELTA_LAUNCH(TT, 4, M); break;                                                                            \
-    case 2: DELTA_LAUNCH(TT, 2, M); break;                                                                            \
-    default: DELTA_LAUNCH(TT, 1, M);                                                                                  \
+  DELTA_CASE(TT, M, 64, 1) DELTA_CASE(TT, M, 64, 2) DELTA_CASE(TT, M, 64, 4) DELTA_CASE(TT, M, 64, 8)                 \
+  DELTA_CASE(TT, M, 128, 2) DELTA_CASE(TT, M, 128, 4) DELTA_CASE(TT, M, 128, 8) DELTA_CASE(TT, M, 128, 16)            \
+  DELTA_CASE(TT, M, 256, 4) DELTA_CASE(TT, M, 256, 8) DELTA_CASE(TT, M, 256, 16) { return -1; }
+  // a whole walk keeps to a wave a SIMD; segments, whose waves hold less, to two. The summaries walk P + D columns.
+#define DELTA_RUN(M)                                                                                                  \
+  {                                                                                                                   \
+    const int lpc = lanes_per_column(D, walks, H, M == 1 ? P + D : P, M == 0 ? 1024 : 2048);                          \
+    if (is_f32) { DELTA_PICK(float, M) } else { DELTA_PICK(bf16_t, M) }                                               \
   }
-#define DELTA_RUN(M) if (is_f32) { DELTA_PICK(float, M) } else { DELTA_PICK(bf16_t, M) }
-  const int lpc = lanes_per_column(D, walks, H, P);
+  const int maxn = D > 128 ? 256 : (D > 64 ? 128 : 64);
   if (!cut) {
     DELTA_RUN(0)
   } else {
@@ -315,6 +318,7 @@ DRYFT_API int dryft_delta_steps(const void* qkv, int64_t qkv_stride, int q_col, 
   }
 #undef DELTA_RUN
 #undef DELTA_PICK
+#undef DELTA_CASE
 #undef DELTA_LAUNCH
   return DRYFT_LAUNCH_CHECK();
 }

@@ -29,7 +29,7 @@ __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log
 // kernel walks a sequence's segments and leaves each the state that enters it; MODE 2 starts every segment from that
 // state and writes its read-outs, and a sequence's last segment writes the state back. Segment x of the step belongs
 // to the sequence s with seg_cu[s] <= x < seg_cu[s + 1] (prefix sums over the sequences; one that sits out has none).
-template <typename T, int LPC, int MODE>
+template <typename T, int LPC, int MODE, int MAXN>
 __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     const T* __restrict__ xbc, int64_t xbc_stride, int x_col, int b_col, int c_col, const float* __restrict__ dt_raw,
     int64_t dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
@@ -38,14 +38,14 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     const int* __restrict__ seg_cu, int n_seqs, int seg_rows, float* __restrict__ seg_state,
     float* __restrict__ seg_decay) {
   constexpr int CW = WAVE / LPC;                       // columns a wave owns
-  constexpr int ROWS = SSM_MAX_STATE / LPC < SSM_ROWS ? SSM_MAX_STATE / LPC : SSM_ROWS;
+  constexpr int ROWS = MAXN / LPC < SSM_ROWS ? MAXN / LPC : SSM_ROWS;
   constexpr int R4 = ROWS / 4;
-  constexpr int PER = SSM_MAX_STATE / 4;               // values of a B or C vector one of its four lanes takes at most
+  constexpr int PER = MAXN / 4;                // values of a B or C vector one of its four lanes takes at most
   constexpr int VN = (SSM_BATCH * CW + WAVE - 1) / WAVE;
   // a vector in LDS: LPC runs (the rows of one lane each), a run padded with zeros to a multiple of 4 floats and
   // followed by 4 more so that neighbouring runs start in different banks
-  __shared__ __attribute__((aligned(16))) float sB[SSM_BATCH][SSM_MAX_STATE + 8 * LPC];
-  __shared__ __attribute__((aligned(16))) float sC[SSM_BATCH][SSM_MAX_STATE + 8 * LPC];
+  __shared__ __attribute__((aligned(16))) float sB[SSM_BATCH][MAXN + 8 * LPC];
+  __shared__ __attribute__((aligned(16))) float sC[SSM_BATCH][MAXN + 8 * LPC];
   __shared__ float sx[SSM_BATCH][CW], sdt[SSM_BATCH], sa[SSM_BATCH];
   const int head = blockIdx.y, p0 = blockIdx.z * CW;
   int seq = blockIdx.x, seg = 0, n_segs = 1;
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(WAVE) void ssm_scan_kernel(
     }
   };
   if (4 * rd4 != rd || rd * LPC != N) {                // what pads the runs stays zero for good
-    for (int i = lane; i < SSM_BATCH * (SSM_MAX_STATE + 8 * LPC); i += WAVE) { (&sB[0][0])[i] = 0.f; (&sC[0][0])[i] = 0.f; }
+    for (int i = lane; i < SSM_BATCH * (MAXN + 8 * LPC); i += WAVE) { (&sB[0][0])[i] = 0.f; (&sC[0][0])[i] = 0.f; }
     __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
@@ -235,13 +235,13 @@ __global__ __launch_bounds__(256) void gate_part_norm_kernel(const float* __rest
 DRYFT_API int dryft_ssm_max_state() { return SSM_MAX_STATE; }
 
 // Lanes a column: as few as hold its rows (64 each), then more while every lane keeps eight rows or more and the
-// launch stays within a wave per SIMD of the chip.
-static int lanes_per_column(int rows_of_state, int n_seqs, int heads, int columns) {
+// launch stays within `most` waves.
+static int lanes_per_column(int rows_of_state, int walks, int heads, int columns, int most) {
   int lpc = rows_of_state > 128 ? 4 : (rows_of_state > 64 ? 2 : 1);
   while (lpc < 16) {
     const int next = 2 * lpc, cw = WAVE / next;
     if ((rows_of_state + next - 1) / next < 8) break;
-    if ((int64_t)n_seqs * heads * ((columns + cw - 1) / cw) > 1024 && cw < columns) break;
+    if ((int64_t)walks * heads * ((columns + cw - 1) / cw) > most && cw < columns) break;
     lpc = next;
   }
   return lpc;
@@ -259,21 +259,22 @@ DRYFT_API int dryft_ssm_scan(const void* xbc, int64_t xbc_stride, int x_col, int
   const int walks = cut ? max_segs : n_seqs;
   // 16-byte loads of B and C: a lane's quarter of a vector in whole pieces of 8 values, at aligned addresses
   const int vec8 = (N % 32 == 0 && b_col % 8 == 0 && c_col % 8 == 0 && xbc_stride % 8 == 0 && ((uintptr_t)xbc & 15) == 0) ? 1 : 0;
-#define SSM_LAUNCH(TT, L, M)                                                                                          \
-  hipLaunchKernelGGL((ssm_scan_kernel<TT, L, M>), dim3(walks, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0, stream, \
+  // The kernel is built for states of up to 64, 128 and 256 rows (X), so that a lane's registers and the loops over
+  // them fit the state at hand.
+#define SSM_LAUNCH(TT, L, M, X)                                                                                       \
+  hipLaunchKernelGGL((ssm_scan_kernel<TT, L, M, X>), dim3(walks, H, (P + WAVE / L - 1) / (WAVE / L)), dim3(WAVE), 0, stream, \
                      (const TT*)xbc, xbc_stride, x_col, b_col, c_col, dt_raw, dt_stride, dt_bias, a_log, d_skip,      \
                      seq_slot, cu_rows, q_len, state, y, H, P, N, G, write_state, vec8, seg_cu, n_seqs, seg_rows,     \
                      seg_state, seg_decay)
+#define SSM_CASE(TT, M, X, L) if (maxn == X && lpc == L) { SSM_LAUNCH(TT, L, M, X); } else
 #define SSM_PICK(TT, M)                                                                                               \
-  switch (lpc) {                                                                                                      \
-    case 16: SSM_LAUNCH(TT, 16, M); break;                                                                            \
-    case 8: SSM_LAUNCH(TT, 8, M); break;                                                                              \
-    case 4: SSM_LAUNCH(TT, 4, M); break;                                                                              \
-    case 2: SSM_LAUNCH(TT, 2, M); break;                                                                              \
-    default: SSM_LAUNCH(TT, 1, M);                                                                                    \
-  }
+  SSM_CASE(TT, M, 64, 1) SSM_CASE(TT, M, 64, 2) SSM_CASE(TT, M, 64, 4) SSM_CASE(TT, M, 64, 8)                         \
+  SSM_CASE(TT, M, 128, 2) SSM_CASE(TT, M, 128, 4) SSM_CASE(TT, M, 128, 8) SSM_CASE(TT, M, 128, 16)                    \
+  SSM_CASE(TT, M, 256, 4) SSM_CASE(TT, M, 256, 8) SSM_CASE(TT, M, 256, 16) { return -1; }
 #define SSM_RUN(M) if (is_f32) { SSM_PICK(float, M) } else { SSM_PICK(bf16_t, M) }
-  const int lpc = lanes_per_column(N, walks, H, P);
+  // a whole walk keeps to a wave a SIMD; segments, whose waves hold less, to two
+  const int maxn = N > 128 ? 256 : (N > 64 ? 128 : 64);
+  const int lpc = lanes_per_column(N, walks, H, P, cut ? 2048 : 1024);
   if (!cut) {
     SSM_RUN(0)
   } else {
@@ -284,6 +285,7 @@ DRYFT_API int dryft_ssm_scan(const void* xbc, int64_t xbc_stride, int x_col, int
   }
 #undef SSM_RUN
 #undef SSM_PICK
+#undef SSM_CASE
 #undef SSM_LAUNCH
   return DRYFT_LAUNCH_CHECK();
 }
