@@ -213,11 +213,12 @@ __global__ __launch_bounds__(WAVE) void delta_steps_kernel(
 }
 
 // The state that enters each segment of a sequence: S_in[0] is the sequence's own state, S_in[s + 1] =
-// A[s] S_in[s] + L[s]. One workgroup per (sequence, head, 8 columns), a thread a row of the state: the columns'
+// A[s] S_in[s] + L[s]. One workgroup per (sequence, head, 4 columns), a thread a row of the state: the columns'
 // current values wait in LDS, every thread reads them all (broadcasts) against its row of A (`seg_trans` holds A
-// column by column, so that the threads of a wave read neighbouring words). `seg_state` holds L when the kernel
-// starts and S_in when it ends.
-#define DELTA_CARRY_COLS 8
+// column by column, so that the threads of a wave read neighbouring words). The walk over a sequence's segments is a
+// chain of dependent steps whose loads of A are what it waits for: few columns a workgroup (many workgroups) and many
+// loads in flight a thread measured best. `seg_state` holds L when the kernel starts and S_in when it ends.
+#define DELTA_CARRY_COLS 4
 __global__ __launch_bounds__(DELTA_MAX_DIM) void delta_carry_kernel(
     const int* __restrict__ seq_slot, const int* __restrict__ seg_cu, const float* __restrict__ state,
     float* __restrict__ seg_state, const float* __restrict__ seg_trans, int H, int D, int P) {
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(DELTA_MAX_DIM) void delta_carry_kernel(
       }
       if (!last) {
         const float* a_row = seg_trans + (((int64_t)(x0 + s)) * H + head) * D * D + d;
-#pragma unroll 8
+#pragma unroll 32
         for (int e = 0; e < D; ++e) {
           const float a = a_row[(int64_t)e * D];
 #pragma unroll

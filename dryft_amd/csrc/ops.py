@@ -92,7 +92,7 @@ _SIGNATURES = {
             "dryft_moe_table_route": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
             "dryft_moe_combine": [_P, _P, _P, _P, _P, _L, _I, _P, _I, _I, _I, _I, _P]},
     "conv": {"dryft_conv_max_taps": [],
-             "dryft_causal_conv": [_P, _L, _I, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+             "dryft_causal_conv": [_P, _L, _I, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
              "dryft_conv_tail": [_P, _L, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _P]},
     "ssm": {"dryft_ssm_max_state": [],
             "dryft_ssm_scan": [_P, _L, _I, _I, _I, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I,
@@ -1763,11 +1763,13 @@ def _row_facts(rows: int, **tensors) -> None:
 
 
 def causal_conv(u, col: int, channels: int, in_bias, weight, out_bias, silu: bool, row_slot, row_seq, row_pos, seq_start,
-                tail, out) -> torch.Tensor:
+                tail, out, weight_t=None) -> torch.Tensor:
     """``out[t, c] = act(sum_j weight[c, j] * v[t - taps + 1 + j, c] + out_bias[c])`` with ``v = u[:, col + c] + in_bias[c]``
     over each sequence's own rows, the ``taps - 1`` inputs before the step's first row from ``tail [slots, taps - 1,
     channels]`` (float32), zeros before the sequence's start. ``act`` is the identity or (``silu``) ``z sigmoid(z)``.
-    Rows of sequences that sit out give zeros. The tail is not touched (``conv_tail`` moves it on)."""
+    Rows of sequences that sit out give zeros. The tail is not touched (``conv_tail`` moves it on). With ``weight_t``
+    (the same weights as contiguous float32 ``[taps, channels]``) and rows that start at multiples of 8 channels a thread
+    takes 8 channels at a time."""
     _gpu(u, "u")
     rows = u.shape[0]
     if not (u.dim() == 2 and u.stride(1) == 1 and 0 <= col and col + channels <= u.shape[1]):
@@ -1777,6 +1779,10 @@ def causal_conv(u, col: int, channels: int, in_bias, weight, out_bias, silu: boo
             1 <= weight.shape[1] <= CONV_MAX_TAPS):
         raise KernelError(f"causal_conv: weight must be contiguous float32 [channels, 1..{CONV_MAX_TAPS}]")
     taps = weight.shape[1]
+    if weight_t is not None:
+        _gpu(weight_t, "weight_t", torch.float32)
+        if not (weight_t.shape == (taps, channels) and weight_t.is_contiguous()):
+            raise KernelError(f"causal_conv: weight_t must be contiguous float32 [{taps}, {channels}]")
     for name, t in (("in_bias", in_bias), ("out_bias", out_bias)):
         if t is not None:
             _f32_vector(t, name, channels)
@@ -1789,7 +1795,8 @@ def causal_conv(u, col: int, channels: int, in_bias, weight, out_bias, silu: boo
     _gpu(out, "out", u.dtype)
     if not (out.shape == (rows, channels) and out.is_contiguous()):
         raise KernelError("causal_conv: out must be contiguous [rows, channels]")
-    _check(_fn("conv", "dryft_causal_conv")(_ptr(u), u.stride(0), col, _ptr(in_bias), _ptr(weight), _ptr(out_bias), taps,
+    _check(_fn("conv", "dryft_causal_conv")(_ptr(u), u.stride(0), col, _ptr(in_bias), _ptr(weight), _ptr(weight_t),
+                                            _ptr(out_bias), taps,
                                             1 if silu else 0, _ptr(row_slot), _ptr(row_seq), _ptr(row_pos),
                                             _ptr(seq_start), _ptr(tail) if taps > 1 else 0, _ptr(out), rows, channels,
                                             _float_flag(u, "u"), _stream()), "causal_conv")

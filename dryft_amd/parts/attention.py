@@ -86,7 +86,7 @@ class GQAAttention(Mixer):
                              self.float_weights or self.has_bias or self.conv_taps)
         self.conv_channels = self.q_dim + self.kv_dim + self.v_dim
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.sink = None
-        self.in_bias = self.o_bias = self.conv_w = None
+        self.in_bias = self.o_bias = self.conv_w = self.conv_wt = None
 
     def tensor_specs(self):
         specs = {"q_proj": matrix((self.q_dim, self.hidden)), "k_proj": matrix((self.kv_dim, self.hidden)),
@@ -123,6 +123,8 @@ class GQAAttention(Mixer):
             self.conv_w = torch.cat([tensors[n].float() for n in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
         elif self.has_bias:                   # the biases ride on a convolution of one tap
             self.conv_w = torch.ones((self.conv_channels, 1), dtype=torch.float32, device=self.in_bias.device)
+        if self.conv_w is not None:
+            self.conv_wt = self.conv_w.t().contiguous()                  # tap by tap, for 8 channels a thread
 
     def cache_need(self):
         kv = KVNeed(self.n_kv, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else None)
@@ -155,7 +157,8 @@ class GQAAttention(Mixer):
         src = proj
         if self.conv_w is not None:
             # biases and the short convolution: q | k | v as one run of channels, each with its own history
-            src = short_conv(proj, 0, self.conv_channels, self.conv_w, ctx, tail, writes_cache, in_bias=self.in_bias)
+            src = short_conv(proj, 0, self.conv_channels, self.conv_w, ctx, tail, writes_cache, in_bias=self.in_bias,
+                             weight_t=self.conv_wt)
         q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
         if isinstance(table, PairRotaryPositions):
             if self.qk_norm_eps is not None:

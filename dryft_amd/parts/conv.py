@@ -21,14 +21,15 @@ def conv_need(taps: int, channels: int) -> StateNeed | None:
 
 
 def short_conv(u: torch.Tensor, col: int, channels: int, weight: torch.Tensor, ctx: StepContext, tail_line,
-               writes_cache: bool, *, in_bias=None, out_bias=None, silu: bool = False) -> torch.Tensor:
+               writes_cache: bool, *, in_bias=None, out_bias=None, silu: bool = False, weight_t=None) -> torch.Tensor:
     """The convolution of columns ``col .. col + channels`` of ``u`` over this step's rows, ``[rows, channels]`` in the
-    dtype of ``u``; ``weight`` is float32 ``[channels, taps]``. With ``writes_cache`` the sequences' tails move on."""
+    dtype of ``u``; ``weight`` is float32 ``[channels, taps]``, ``weight_t`` (optional) the same tap by tap, ``[taps,
+    channels]``, for the kernel that takes 8 channels a thread. With ``writes_cache`` the sequences' tails move on."""
     taps = weight.shape[1]
     tail = tail_line.state if taps > 1 else None
     out = torch.empty((u.shape[0], channels), dtype=u.dtype, device=u.device)
     ops.causal_conv(u, col, channels, in_bias, weight, out_bias, silu, ctx.row_slot, ctx.row_seq, ctx.row_pos,
-                    ctx.seq_start, tail, out)
+                    ctx.seq_start, tail, out, weight_t=weight_t)
     if writes_cache and taps > 1:
         ops.conv_tail(u, col, channels, in_bias, taps, ctx.seq_slot, ctx.cu_rows, ctx.q_len, ctx.n_seqs, tail)
     return out

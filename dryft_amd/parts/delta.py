@@ -62,6 +62,7 @@ class GatedDeltaMixer(Mixer):
         self.w_gates = torch.cat([tensors["a_proj"], tensors["b_proj"]], dim=0).contiguous()
         self.w_o = tensors["o_proj"]
         self.conv_w = torch.cat([tensors[n].float() for n in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.conv_wt = self.conv_w.t().contiguous()                         # tap by tap, for 8 channels a thread
         self.dt_bias, self.a_log = tensors["dt_bias"].float().contiguous(), tensors["a_log"].float().contiguous()
         self.out_norm = tensors["out_norm"].float().repeat(self.n_heads).contiguous()      # one weight for every head
 
@@ -78,7 +79,8 @@ class GatedDeltaMixer(Mixer):
         rows = h.shape[0]
         proj = linear(h, self.w_in)                                        # q | k | v | gate, in the activation dtype
         gates = linear(h, self.w_gates, out_dtype=torch.float32)            # a | b stay float32 from here on
-        qkv = short_conv(proj, 0, self.conv_channels, self.conv_w, ctx, line.get("tail"), writes_cache, silu=True)
+        qkv = short_conv(proj, 0, self.conv_channels, self.conv_w, ctx, line.get("tail"), writes_cache, silu=True,
+                         weight_t=self.conv_wt)
         # the rows of sequences that sit out are not visited by the walk; the read-out norms whatever they hold
         o_raw = ctx.kept_zeros((rows, self.v_dim), torch.float32) if ctx.some_sit_out() else \
             torch.empty((rows, self.v_dim), dtype=torch.float32, device=h.device)

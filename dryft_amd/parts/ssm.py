@@ -64,6 +64,7 @@ class StateSpaceMixer(Mixer):
         self.w_dt = w[cut:].contiguous()              # the step sizes: their product keeps its float32 accumulators
         self.w_o = tensors["o_proj"]
         self.conv_w, self.conv_b = tensors["conv"].float().contiguous(), tensors["conv_bias"].float().contiguous()
+        self.conv_wt = self.conv_w.t().contiguous()
         for name in ("dt_bias", "a_log", "d_skip", "out_norm"):
             setattr(self, name, tensors[name].float().contiguous())
 
@@ -81,7 +82,7 @@ class StateSpaceMixer(Mixer):
         proj = linear(h, self.w_in)
         dt_raw = linear(h, self.w_dt, out_dtype=torch.float32)
         xbc = short_conv(proj, self.inner, self.conv_channels, self.conv_w, ctx, line.get("tail"), writes_cache,
-                         out_bias=self.conv_b, silu=True)
+                         out_bias=self.conv_b, silu=True, weight_t=self.conv_wt)
         # a long prompt runs as segments side by side (the rows of sequences that sit out are then not visited)
         segments = ctx.segments() if writes_cache else None
         y = torch.empty((rows, self.inner), dtype=torch.float32, device=h.device)

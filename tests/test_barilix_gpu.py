@@ -87,10 +87,11 @@ def test_scaled_embedding_starts_a_float_stream(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("taps,channels", [(1, 24), (2, 300), (4, 64), (7, 9)])
-def test_short_convolution_and_its_tail(dtype, taps, channels):
+@pytest.mark.parametrize("taps,channels,col", [(1, 24, 8), (2, 300, 5), (4, 64, 5), (7, 9, 5), (4, 64, 8), (3, 136, 16)])
+def test_short_convolution_and_its_tail(dtype, taps, channels, col):
     """The kernel pair alone, through steps of every size: what the tail holds after a step is what the next one reads,
-    also where a step brings fewer rows than the tail is long, and a slot that is freed starts from zeros again."""
+    also where a step brings fewer rows than the tail is long, and a slot that is freed starts from zeros again. Channels
+    that start at a multiple of 8 columns take the kernel of 8 channels a thread, the others the one of a channel."""
     from dryft_amd.cache import CacheStore
     from dryft_amd.engine.step import BatchBuffers, stage_batch
     from dryft_amd.parts.conv import conv_need, short_conv
@@ -101,7 +102,7 @@ def test_short_convolution_and_its_tail(dtype, taps, channels):
     weight, in_bias, out_bias = torch.randn(channels, taps, generator=g), torch.randn(channels, generator=g), torch.randn(channels, generator=g)
     buf = BatchBuffers(512, 4, DEV)
     for attempt in range(2):                                  # the second time in slots that were used before
-        seqs = [torch.randn(n, channels + 5, generator=g).to(T) for n in (40, 3, 17)]
+        seqs = [torch.randn(n, channels + col, generator=g).to(T) for n in (40, 3, 17)]
         slots = cache.acquire(3)
         got = [[] for _ in seqs]
         for cuts in ([1, 2, 3, 4, 6, 9, 30],):
@@ -112,8 +113,9 @@ def test_short_convolution_and_its_tail(dtype, taps, channels):
                 ctx = stage_batch(cache, buf, [slots[i] for i, _ in live], q_lens, [0] * sum(q_lens), T)
                 u = torch.cat([x for _, x in live]).to(DEV)
                 line = cache.line(0)
-                out = short_conv(u, 5, channels, weight.to(DEV), ctx, line["tail"] if line else None, True,
-                                 in_bias=in_bias.to(DEV), out_bias=out_bias.to(DEV), silu=True)
+                out = short_conv(u, col, channels, weight.to(DEV), ctx, line["tail"] if line else None, True,
+                                 in_bias=in_bias.to(DEV), out_bias=out_bias.to(DEV), silu=True,
+                                 weight_t=weight.t().contiguous().to(DEV) if col % 8 == 0 else None)
                 cache.end_step([slots[i] for i, _ in live], q_lens)
                 at = 0
                 for i, x in live:
@@ -121,7 +123,7 @@ def test_short_convolution_and_its_tail(dtype, taps, channels):
                     at += len(x)
         cache.release(slots)
         for s, mine in zip(seqs, got):
-            want = P.silu(P.short_conv(s.double()[:, 5:] + in_bias.double(), weight.double(), None, out_bias.double())[0])
+            want = P.silu(P.short_conv(s.double()[:, col:] + in_bias.double(), weight.double(), None, out_bias.double())[0])
             assert rel_err(torch.cat(mine), want) <= (2e-6 if dtype == "float32" else 8e-3), (taps, attempt)
 
 
