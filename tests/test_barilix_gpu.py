@@ -102,11 +102,11 @@ def test_short_convolution_and_its_tail(dtype, taps, channels, col):
     weight, in_bias, out_bias = torch.randn(channels, taps, generator=g), torch.randn(channels, generator=g), torch.randn(channels, generator=g)
     buf = BatchBuffers(512, 4, DEV)
     for attempt in range(2):                                  # the second time in slots that were used before
-        seqs = [torch.randn(n, channels + col, generator=g).to(T) for n in (40, 3, 17)]
+        seqs = [torch.randn(n, channels + col, generator=g).to(T) for n in (120, 3, 57)]
         slots = cache.acquire(3)
         got = [[] for _ in seqs]
         for cuts in ([1, 2, 3, 4, 6, 9, 30],):
-            edges = [0] + cuts + [40]
+            edges = [0] + cuts + [120]               # steps of few rows, then one of many (another kernel)
             for a, b in zip(edges[:-1], edges[1:]):
                 live = [(i, s[a:b]) for i, s in enumerate(seqs) if len(s[a:b])]
                 q_lens = [len(x) for _, x in live]
