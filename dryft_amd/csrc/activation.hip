@@ -125,3 +125,80 @@ DRYFT_API int dryft_sigmoid_gate(const void* a, int64_t a_stride, const void* g,
                        (const bf16_t*)g, g_stride, (bf16_t*)y, width);
   return DRYFT_LAUNCH_CHECK();
 }
+
+// The square of relu: y = T( max(x, 0)^2 ), rows of `width` values; x may be a run of columns of a wider tensor.
+template <typename T>
+__global__ void relu_squared_kernel(const T* __restrict__ x, int64_t x_stride, T* __restrict__ y, int width) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  const float r = fmaxf(load_as_float(x + row * x_stride + i), 0.f);
+  store_from_float(y + row * width + i, r * r);
+}
+
+DRYFT_API int dryft_relu_squared(const void* x, int64_t x_stride, void* y, int n_rows, int width, int is_f32,
+                                 hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  dim3 grid(n_rows, (width + 255) / 256), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(relu_squared_kernel<float>, grid, block, 0, stream, (const float*)x, x_stride, (float*)y, width);
+  else
+    hipLaunchKernelGGL(relu_squared_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)x, x_stride, (bf16_t*)y, width);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// A gate on what a token id brings: y[r, i] = T( gelu_tanh(g[r, i]) * table[token[r], col + i] ), with
+// gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))); the table's row is as wide as the caller says.
+template <typename T>
+__global__ void token_gate_kernel(const T* __restrict__ g, int64_t g_stride, const int* __restrict__ tokens,
+                                  const T* __restrict__ table, int64_t table_stride, int col, int vocab,
+                                  T* __restrict__ y, int width) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  const int tok = min(max(tokens[row], 0), vocab - 1);
+  const float z = load_as_float(g + row * g_stride + i);
+  const float act = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  store_from_float(y + row * width + i, act * load_as_float(table + (int64_t)tok * table_stride + col + i));
+}
+
+DRYFT_API int dryft_token_gate(const void* g, int64_t g_stride, const int* tokens, const void* table,
+                               int64_t table_stride, int col, int vocab, void* y, int n_rows, int width, int is_f32,
+                               hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (vocab <= 0 || col < 0 || col + width > table_stride) return -1;
+  dim3 grid(n_rows, (width + 255) / 256), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(token_gate_kernel<float>, grid, block, 0, stream, (const float*)g, g_stride, tokens,
+                       (const float*)table, table_stride, col, vocab, (float*)y, width);
+  else
+    hipLaunchKernelGGL(token_gate_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)g, g_stride, tokens,
+                       (const bf16_t*)table, table_stride, col, vocab, (bf16_t*)y, width);
+  return DRYFT_LAUNCH_CHECK();
+}
+
+// A blend of two runs of columns, in place: a[r, i] = T( (1 - lam) a[r, i] + lam b[r, i] ), lam one float on the
+// device. Float arithmetic, rounded once.
+template <typename T>
+__global__ void blend_columns_kernel(T* __restrict__ a, int64_t a_stride, const T* __restrict__ b, int64_t b_stride,
+                                     const float* __restrict__ lam, int width) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  const float l = *lam;
+  T* p = a + row * a_stride + i;
+  store_from_float(p, (1.f - l) * load_as_float(p) + l * load_as_float(b + row * b_stride + i));
+}
+
+DRYFT_API int dryft_blend_columns(void* a, int64_t a_stride, const void* b, int64_t b_stride, const float* lam,
+                                  int n_rows, int width, int is_f32, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  dim3 grid(n_rows, (width + 255) / 256), block(256);
+  if (is_f32)
+    hipLaunchKernelGGL(blend_columns_kernel<float>, grid, block, 0, stream, (float*)a, a_stride, (const float*)b,
+                       b_stride, lam, width);
+  else
+    hipLaunchKernelGGL(blend_columns_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)a, a_stride, (const bf16_t*)b,
+                       b_stride, lam, width);
+  return DRYFT_LAUNCH_CHECK();
+}

@@ -12,7 +12,10 @@
 // Options that other designs use: a value width v_dim that differs from the key width; a capped score,
 // s <- cap * tanh(s / cap); a sink, one learned number per query head whose exp() joins the softmax's
 // denominator and nothing else (no key, no value; neither scaled nor capped); probabilities kept in
-// float (exact_p), for designs that ask for float attention weights also in bfloat16.
+// float (exact_p), for designs that ask for float attention weights also in bfloat16; chunks, where a row sees
+// the keys of its own run of `chunk` positions only (runs counted from position 0: lo = pos - pos % chunk); and a
+// learned bias by distance, rel[min(pos - j, n_dist - 1)][head] (float32, one row per distance, the last row for
+// every larger one), added to the scaled score.
 #include "common.h"
 
 #define ROWS_THREADS 256
@@ -23,7 +26,8 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
                                  const int* __restrict__ page_table, int max_pages, const int* __restrict__ row_slot,
                                  const int* __restrict__ row_pos, T* __restrict__ out, int n_heads, int n_kv,
                                  int head_dim, int v_dim, float scale, int window, float softcap,
-                                 const float* __restrict__ sink, int exact_p, int vec) {
+                                 const float* __restrict__ sink, int exact_p, int vec, int chunk,
+                                 const float* __restrict__ rel, int n_dist) {
   __shared__ float qs[ROWS_MAX_HEAD_DIM];
   __shared__ float ps[ROWS_THREADS];
   __shared__ int pages[ROWS_THREADS / PAGE_TOKENS];
@@ -38,7 +42,7 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
   }
   const int pos = row_pos[row];
   const int kvh = head / (n_heads / n_kv);
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = chunk > 0 ? pos - pos % chunk : (window > 0 ? max(0, pos - window + 1) : 0);
   if (tid < head_dim) qs[tid] = load_as_float(q + (row * n_heads + head) * head_dim + tid);
   float m = -INFINITY, l = 0.f, acc = 0.f;
   for (int c = (lo / PAGE_TOKENS) * PAGE_TOKENS; c <= pos; c += ROWS_THREADS) {
@@ -67,6 +71,7 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
       }
       s = d * scale;
       if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+      if (rel != nullptr) s += rel[(int64_t)min(pos - j, n_dist - 1) * n_heads + head];
     }
     const float m_new = fmaxf(m, block_max(s, scratch));  // finite: every chunk holds a key the row sees
     const float alpha = expf(m - m_new);                   // first chunk: exp(-inf) = 0
@@ -122,18 +127,20 @@ __global__ void attn_rows_kernel(const T* __restrict__ q, const T* __restrict__ 
 DRYFT_API int dryft_attn_rows(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                               int max_pages, const int* row_slot, const int* row_pos, void* out, int n_rows,
                               int n_heads, int n_kv, int head_dim, int v_dim, float scale, int window, float softcap,
-                              const float* sink, int exact_p, int is_f32, hipStream_t stream) {
+                              const float* sink, int exact_p, int chunk, const float* rel, int n_dist, int is_f32,
+                              hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (chunk < 0 || (rel != nullptr && n_dist <= 0)) return -1;
   if (head_dim > ROWS_MAX_HEAD_DIM || v_dim <= 0 || v_dim > ROWS_THREADS || n_kv <= 0 || n_heads % n_kv) return -1;
   dim3 grid(n_rows, n_heads), block(ROWS_THREADS);
   const int vec = head_dim % 8 == 0 && v_dim % 8 == 0 && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0;
   if (is_f32)
     hipLaunchKernelGGL(attn_rows_kernel<float>, grid, block, 0, stream, (const float*)q, (const float*)k_pages,
                        (const float*)v_pages, page_table, max_pages, row_slot, row_pos, (float*)out, n_heads, n_kv,
-                       head_dim, v_dim, scale, window, softcap, sink, exact_p, vec);
+                       head_dim, v_dim, scale, window, softcap, sink, exact_p, vec, chunk, rel, n_dist);
   else
     hipLaunchKernelGGL(attn_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, (const bf16_t*)k_pages,
                        (const bf16_t*)v_pages, page_table, max_pages, row_slot, row_pos, (bf16_t*)out, n_heads, n_kv,
-                       head_dim, v_dim, scale, window, softcap, sink, exact_p, vec);
+                       head_dim, v_dim, scale, window, softcap, sink, exact_p, vec, chunk, rel, n_dist);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -46,7 +46,8 @@ DRYFT_API int dryft_rms_segments(const void* src, int64_t stride, int col, const
 //
 //   o[i] = x[i] c - x[i + rot/2] s,   o[i + rot/2] = x[i + rot/2] c + x[i] s,   c, s = cos, sin of pos * f_i
 //
-// in float with float32 tables [positions, rot/2], rounded once; the rest passes. Keys go to pages [64][key_dim],
+// in float with float32 tables [positions, rot/2], rounded once; the rest passes. With `pairs` feature 2i turns
+// with feature 2i + 1 instead (the same tables, angle i for pair i). Keys go to pages [64][key_dim],
 // values transposed to pages [page_dv][64] in the kernels' column order (rows from value_dim on are never
 // written and stay zero). One wave per (row, head) of q, k and v.
 template <typename T>
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(256) void latent_rope_kv_kernel(
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, const int* __restrict__ row_slot,
     const int* __restrict__ row_pos, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, int write_kv, int n_heads, int plain, int rot_dim, int v_dim,
-    int page_dv) {
+    int page_dv, int pairs) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t row = blockIdx.x;
   const int job = blockIdx.y * 4 + wave;
@@ -88,9 +89,10 @@ __global__ __launch_bounds__(256) void latent_rope_kv_kernel(
   const int half = rot / 2;
   for (int i = lane; i < half; i += WAVE) {
     const float c = cos_t[(int64_t)pos * half + i], s = sin_t[(int64_t)pos * half + i];
-    const float a = load_as_float(src_rot + i), b = load_as_float(src_rot + half + i);
-    store_from_float(dst + plain + i, a * c - b * s);
-    store_from_float(dst + plain + half + i, b * c + a * s);
+    const int ia = pairs ? 2 * i : i, ib = pairs ? 2 * i + 1 : half + i;
+    const float a = load_as_float(src_rot + ia), b = load_as_float(src_rot + ib);
+    store_from_float(dst + plain + ia, a * c - b * s);
+    store_from_float(dst + plain + ib, b * c + a * s);
   }
   for (int i = rot + lane; i < rot_dim; i += WAVE) dst[plain + i] = src_rot[i];
 }
@@ -99,7 +101,7 @@ DRYFT_API int dryft_latent_rope_kv(const void* q_raw, const void* kv, const void
                                    const float* cos_t, const float* sin_t, int rot, const int* row_slot,
                                    const int* row_pos, void* q_out, void* k_pages, void* v_pages, const int* page_table,
                                    int max_pages, int write_kv, int n_rows, int n_heads, int plain, int rot_dim, int v_dim,
-                                   int page_dv, int is_f32, hipStream_t stream) {
+                                   int page_dv, int pairs, int is_f32, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (rot < 0 || rot % 2 || rot > rot_dim || n_heads <= 0 || v_dim > page_dv) return -1;
   dim3 grid(n_rows, (3 * n_heads + 3) / 4), block(256);
@@ -107,42 +109,44 @@ DRYFT_API int dryft_latent_rope_kv(const void* q_raw, const void* kv, const void
     hipLaunchKernelGGL(latent_rope_kv_kernel<float>, grid, block, 0, stream, (const float*)q_raw, (const float*)kv,
                        (const float*)down, down_stride, krot_col, cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out,
                        (float*)k_pages, (float*)v_pages, page_table, max_pages, write_kv, n_heads, plain, rot_dim, v_dim,
-                       page_dv);
+                       page_dv, pairs);
   else
     hipLaunchKernelGGL(latent_rope_kv_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q_raw, (const bf16_t*)kv,
                        (const bf16_t*)down, down_stride, krot_col, cos_t, sin_t, rot, row_slot, row_pos, (bf16_t*)q_out,
                        (bf16_t*)k_pages, (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads, plain, rot_dim,
-                       v_dim, page_dv);
+                       v_dim, page_dv, pairs);
   return DRYFT_LAUNCH_CHECK();
 }
 
 // ---------------------------------------------------------------------------------------------------
 // out[row, head, :v_dim] = attn[row, head, :v_dim] * sigmoid(gate[row, head]); the heads of `attn` may be wider
-// than v_dim (in_dim), `out` is packed. The gate's logits are columns g_col.. of `down`.
+// than v_dim (in_dim), `out` is packed. The gate's logits are columns g_col.. of `down`: one per head, or with
+// `per_element` one per output (head by head, v_dim each).
 template <typename T>
 __global__ __launch_bounds__(256) void head_gate_kernel(const T* __restrict__ attn, const T* __restrict__ down,
                                                         int64_t down_stride, int g_col, T* __restrict__ out,
-                                                        int64_t total, int n_heads, int in_dim, int v_dim) {
+                                                        int64_t total, int n_heads, int in_dim, int v_dim,
+                                                        int per_element) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const int j = idx % v_dim;
   const int64_t rh = idx / v_dim, row = rh / n_heads;
   const int head = rh % n_heads;
-  const float g = load_as_float(down + row * down_stride + g_col + head);
+  const float g = load_as_float(down + row * down_stride + g_col + (per_element ? head * v_dim + j : head));
   store_from_float(out + idx, load_as_float(attn + rh * in_dim + j) / (1.f + expf(-g)));
 }
 
 DRYFT_API int dryft_head_gate(const void* attn, const void* down, int64_t down_stride, int g_col, void* out, int rows,
-                              int n_heads, int in_dim, int v_dim, int is_f32, hipStream_t stream) {
+                              int n_heads, int in_dim, int v_dim, int per_element, int is_f32, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (v_dim > in_dim) return -1;
   const int64_t total = (int64_t)rows * n_heads * v_dim;
   dim3 grid((unsigned)((total + 255) / 256)), block(256);
   if (is_f32)
     hipLaunchKernelGGL(head_gate_kernel<float>, grid, block, 0, stream, (const float*)attn, (const float*)down,
-                       down_stride, g_col, (float*)out, total, n_heads, in_dim, v_dim);
+                       down_stride, g_col, (float*)out, total, n_heads, in_dim, v_dim, per_element);
   else
     hipLaunchKernelGGL(head_gate_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)attn, (const bf16_t*)down,
-                       down_stride, g_col, (bf16_t*)out, total, n_heads, in_dim, v_dim);
+                       down_stride, g_col, (bf16_t*)out, total, n_heads, in_dim, v_dim, per_element);
   return DRYFT_LAUNCH_CHECK();
 }

@@ -28,24 +28,45 @@ __device__ __forceinline__ Best wave_best(Best b) {
 // score is the sum of its two largest choice scores (of its only one, if it has one); experts outside the `keep`
 // best groups drop out. The `top` largest choice scores that remain are chosen, highest first, and weigh
 // s / (sum of the chosen s + 1e-20) * scale. One wave a row; lane l holds experts l, l + 64, ...
+// Other forms: `softmax` takes s = softmax(z) over all experts instead of the sigmoid; no correction (null): the
+// choice scores are s itself; `group_best`: a group scores as its single largest choice score; without `renorm`
+// the weights are s * scale as they are.
 template <int PER>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int64_t stride,
                                                         const float* __restrict__ correction, int n_experts, int groups,
                                                         int keep, int top, float scale, int* __restrict__ chosen,
-                                                        float* __restrict__ weights, int rows) {
+                                                        float* __restrict__ weights, int rows, int softmax,
+                                                        int group_best, int renorm) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;
   if (row >= rows) return;
   const float NEG = -__builtin_inff();
   float s[PER], c[PER];
+  float z_max = NEG, z_sum = 0.f;
+  if (softmax) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + WAVE * j;
+      if (e < n_experts) z_max = fmaxf(z_max, logits[row * stride + e]);
+    }
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) z_max = fmaxf(z_max, __shfl_xor(z_max, o, WAVE));
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + WAVE * j;
+      s[j] = e < n_experts ? expf(logits[row * stride + e] - z_max) : 0.f;
+      z_sum += s[j];
+    }
+    z_sum = wave_sum(z_sum);
+  }
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int e = lane + WAVE * j;
-    s[j] = 0.f;
+    if (!softmax) s[j] = 0.f;
     c[j] = NEG;
     if (e < n_experts) {
-      s[j] = 1.f / (1.f + expf(-logits[row * stride + e]));
-      c[j] = s[j] + correction[e];
+      s[j] = softmax ? s[j] / z_sum : 1.f / (1.f + expf(-logits[row * stride + e]));
+      c[j] = s[j] + (correction != nullptr ? correction[e] : 0.f);
     }
   }
   if (keep < groups) {
@@ -60,7 +81,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
       }
       a = wave_best(a);
       float sum = a.v;
-      if (size >= 2) {
+      if (size >= 2 && !group_best) {
         Best b{NEG, 0x7fffffff};
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
@@ -106,21 +127,23 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
   }
   if (lane == 0)       // the same lane wrote them
-    for (int i = 0; i < top; ++i) weights[row * top + i] = weights[row * top + i] / (total + 1e-20f) * scale;
+    for (int i = 0; i < top; ++i)
+      weights[row * top + i] = renorm ? weights[row * top + i] / (total + 1e-20f) * scale : weights[row * top + i] * scale;
 }
 
 DRYFT_API int dryft_moe_max_experts() { return MOE_MAX_EXPERTS; }
 DRYFT_API int dryft_moe_tile() { return MOE_TILE; }
 
 DRYFT_API int dryft_moe_route(const float* logits, int64_t stride, const float* correction, int n_experts, int groups,
-                              int keep, int top, float scale, int* chosen, float* weights, int rows, hipStream_t stream) {
+                              int keep, int top, float scale, int* chosen, float* weights, int rows, int softmax,
+                              int group_best, int renorm, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (n_experts < 1 || n_experts > MOE_MAX_EXPERTS || top < 1 || top > n_experts || groups < 1 || groups > WAVE ||
       n_experts % groups || keep < 1 || keep > groups || keep * (n_experts / groups) < top)
     return -1;
 #define MOE_ROUTE(PER)                                                                                              \
   hipLaunchKernelGGL(moe_route_kernel<PER>, dim3((rows + 3) / 4), dim3(256), 0, stream, logits, stride, correction,   \
-                     n_experts, groups, keep, top, scale, chosen, weights, rows)
+                     n_experts, groups, keep, top, scale, chosen, weights, rows, softmax, group_best, renorm)
   if (n_experts <= WAVE) MOE_ROUTE(1);
   else if (n_experts <= 2 * WAVE) MOE_ROUTE(2);
   else MOE_ROUTE(MOE_PER_LANE);
@@ -205,7 +228,8 @@ DRYFT_API int dryft_moe_table_route(const int* tokens, const int* table, int* ch
 // otherwise `a` is already in place order. GLU: W_e holds gate rows then up rows; the clamped gated unit
 // g * sigmoid(alpha g) * (u + offset), g = min(gate, limit), u = clamp(up, -limit, limit) (offset 0, alpha 1 and an
 // infinite limit make it silu(gate) * up), is applied to the float
-// accumulators and `n_out` counts its outputs.
+// accumulators and `n_out` counts its outputs. Without a gate, `act` = 1 stores the square of relu of the product
+// (as it would have been stored in the activation dtype) instead of the product.
 #define MOE_TN 64
 #define MOE_TK 32
 
@@ -216,7 +240,7 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
                                                           const int* __restrict__ tile_start,
                                                           const int* __restrict__ tile_rows,
                                                           const int* __restrict__ n_tiles, O* __restrict__ out, int top,
-                                                          int n_out, int k_dim, float limit, float alpha, float offset) {
+                                                          int n_out, int k_dim, float limit, float alpha, float offset, int act) {
   __shared__ float sa[MOE_TILE][MOE_TK + 1];
   __shared__ float sw[(GLU ? 2 : 1) * MOE_TN][MOE_TK + 1];
   __shared__ int src_row[MOE_TILE];
@@ -280,6 +304,9 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
         const float g = fminf(rounded_as<T>(v), limit);
         const float u = fminf(fmaxf(rounded_as<T>(acc_up[i][j]), -limit), limit);
         v = g / (1.f + expf(-alpha * g)) * (u + offset);
+      } else if (act == 1) {
+        const float r = fmaxf(rounded_as<T>(v), 0.f);
+        v = r * r;
       }
       store_from_float(out + (int64_t)(start + r) * n_out + n, v);
     }
@@ -309,7 +336,7 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
                                                                const int* __restrict__ tile_start,
                                                                const int* __restrict__ tile_rows,
                                                                const int* __restrict__ n_tiles, O* __restrict__ out,
-                                                               int top, int n_out, int k_dim, float limit, float alpha, float offset) {
+                                                               int top, int n_out, int k_dim, float limit, float alpha, float offset, int act) {
   constexpr int MT = MOE_TILE / 16;
   __shared__ __attribute__((aligned(16))) bf16_t sx[2][MOE_TILE * MOE_X_STRIDE];
   const int tile = blockIdx.x;
@@ -381,6 +408,9 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(const bf16_t* __r
         const float gv = fminf(rounded_as<bf16_t>(v), limit);
         const float uv = fminf(fmaxf(rounded_as<bf16_t>(acc_up[mt][i]), -limit), limit);
         v = gv / (1.f + expf(-alpha * gv)) * (uv + offset);
+      } else if (act == 1) {
+        const float r = fmaxf(rounded_as<bf16_t>(v), 0.f);
+        v = r * r;
       }
       store_from_float(out + (int64_t)(start + m) * n_out + n, v);
     }
@@ -399,7 +429,7 @@ __global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __re
                                                               const int* __restrict__ tile_start,
                                                               const int* __restrict__ tile_rows,
                                                               const int* __restrict__ n_tiles, O* __restrict__ out,
-                                                              int top, int n_out, int k_dim, float limit, float alpha, float offset) {
+                                                              int top, int n_out, int k_dim, float limit, float alpha, float offset, int act) {
   const int tile = blockIdx.x;
   if (tile >= *n_tiles) return;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, c = lane % 16, g = lane / 16;
@@ -446,6 +476,9 @@ __global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __re
         const float gv = fminf(rounded_as<bf16_t>(v), limit);
         const float uv = fminf(fmaxf(rounded_as<bf16_t>(acc_up[i]), -limit), limit);
         v = gv / (1.f + expf(-alpha * gv)) * (uv + offset);
+      } else if (act == 1) {
+        const float r = fmaxf(rounded_as<bf16_t>(v), 0.f);
+        v = r * r;
       }
       store_from_float(out + (int64_t)(start + m) * n_out + n, v);
     }
@@ -455,7 +488,7 @@ __global__ __launch_bounds__(256) void moe_product_few_kernel(const bf16_t* __re
 DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, const int* sorted_pair,
                                 const int* tile_expert, const int* tile_start, const int* tile_rows, const int* n_tiles,
                                 int max_tiles, void* out, int out_is_f32, int top, int n_out, int k_dim, int glu,
-                                float limit, float alpha, float offset, int most_places, int is_f32, hipStream_t stream) {
+                                float limit, float alpha, float offset, int act, int most_places, int is_f32, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (n_out <= 0 || k_dim <= 0 || (glu && out_is_f32 && !is_f32)) return -1;
   dim3 grid(max_tiles, (n_out + MOE_TN - 1) / MOE_TN), block(256);
@@ -464,7 +497,7 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
 #define MOE_FEW(O, G)                                                                                             \
   hipLaunchKernelGGL((moe_product_few_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,           \
                      (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \
-                     k_dim, limit, alpha, offset)
+                     k_dim, limit, alpha, offset, act)
       if (glu) MOE_FEW(bf16_t, true);
       else if (out_is_f32) MOE_FEW(float, false);
       else MOE_FEW(bf16_t, false);
@@ -474,7 +507,7 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
 #define MOE_MFMA(O, G)                                                                                            \
   hipLaunchKernelGGL((moe_product_mfma_kernel<O, G>), grid, block, 0, stream, (const bf16_t*)a, a_stride,          \
                      (const bf16_t*)w, sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, \
-                     k_dim, limit, alpha, offset)
+                     k_dim, limit, alpha, offset, act)
     if (glu) MOE_MFMA(bf16_t, true);
     else if (out_is_f32) MOE_MFMA(float, false);
     else MOE_MFMA(bf16_t, false);
@@ -483,7 +516,7 @@ DRYFT_API int dryft_moe_product(const void* a, int64_t a_stride, const void* w, 
   }
 #define MOE_LAUNCH(T, O, G)                                                                                       \
   hipLaunchKernelGGL((moe_product_kernel<T, O, G>), grid, block, 0, stream, (const T*)a, a_stride, (const T*)w,   \
-                     sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, k_dim, limit, alpha, offset)
+                     sorted_pair, tile_expert, tile_start, tile_rows, n_tiles, (O*)out, top, n_out, k_dim, limit, alpha, offset, act)
   if (is_f32) {
     if (glu) MOE_LAUNCH(float, float, true); else MOE_LAUNCH(float, float, false);
   } else if (glu) {

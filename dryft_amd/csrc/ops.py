@@ -28,7 +28,10 @@ _SIGNATURES = {
              "dryft_rms_pair_mean": [_P, _I, _I, _L, _P, _P, _P, _I, _I, _L, _P, _P, _P, _I, _I, _F, _I, _P]},
     "activation": {"dryft_silu_mul": [_P, _P, _I, _I, _L, _I, _P],
                    "dryft_glu_clamped": [_P, _P, _I, _I, _L, _F, _F, _I, _P],
-                   "dryft_sigmoid_gate": [_P, _L, _P, _L, _P, _I, _I, _I, _P]},
+                   "dryft_sigmoid_gate": [_P, _L, _P, _L, _P, _I, _I, _I, _P],
+                   "dryft_relu_squared": [_P, _L, _P, _I, _I, _I, _P],
+                   "dryft_token_gate": [_P, _L, _P, _P, _L, _I, _I, _P, _I, _I, _I, _P],
+                   "dryft_blend_columns": [_P, _L, _P, _L, _P, _I, _I, _I, _P]},
     "mlstm": {"dryft_mlstm_steps": [_P, _L, _I, _I, _I, _P, _P, _P, _F, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _F,
                                     _I, _I, _P],
               "dryft_mlstm_chunks_takes": [_I, _I, _I, _I, _I, _L],
@@ -50,7 +53,7 @@ _SIGNATURES = {
                 "dryft_rows_to_cache_takes": [_I, _I, _I, _I],
                 "dryft_rows_to_cache_parts": [_P, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                               _I, _I, _I, _P]},
-    "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P, _I, _I, _P]},
+    "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P, _I, _I, _P, _I, _I, _P]},
     "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _I, _F, _P,
                                              _P],
                   "dryft_attn_causal_takes_projection": [_I, _I],
@@ -84,11 +87,11 @@ _SIGNATURES = {
             "dryft_wkv_out": [_P, _P, _P, _P, _I, _I, _I, _F, _L, _I, _P]},
     "latent": {"dryft_rms_segments": [_P, _L, _I, _P, _P, _I, _P, _P, _I, _F, _I, _I, _P],
                "dryft_latent_rope_kv": [_P, _P, _P, _L, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
-                                        _I, _I, _I, _P],
-               "dryft_head_gate": [_P, _P, _L, _I, _P, _I, _I, _I, _I, _I, _P]},
-    "moe": {"dryft_moe_route": [_P, _L, _P, _I, _I, _I, _I, _F, _P, _P, _I, _P],
+                                        _I, _I, _I, _I, _P],
+               "dryft_head_gate": [_P, _P, _L, _I, _P, _I, _I, _I, _I, _I, _I, _P]},
+    "moe": {"dryft_moe_route": [_P, _L, _P, _I, _I, _I, _I, _F, _P, _P, _I, _I, _I, _I, _P],
             "dryft_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P],
-            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _F, _I, _I, _P],
+            "dryft_moe_product": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _F, _I, _I, _I, _P],
             "dryft_moe_table_route": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
             "dryft_moe_combine": [_P, _P, _P, _P, _P, _L, _I, _P, _I, _I, _I, _I, _P]},
     "conv": {"dryft_conv_max_taps": [],
@@ -349,6 +352,49 @@ def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor, out: torch.Tensor) -> torc
     return out
 
 
+def relu_squared(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out = max(x, 0)^2``; ``x`` is ``[rows, width]`` and may be a column run of a wider tensor."""
+    _gpu(x, "x")
+    _gpu(out, "out", x.dtype)
+    rows, width = x.shape
+    if not (x.stride(1) == 1 and out.shape == x.shape and out.is_contiguous()):
+        raise KernelError("relu_squared: x [rows, width] with unit column stride, out contiguous")
+    _check(_fn("activation", "dryft_relu_squared")(_ptr(x), x.stride(0), _ptr(out), rows, width, _float_flag(x, "x"),
+                                                   _stream()), "relu_squared")
+    return out
+
+
+def token_gate(gate: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col: int, out: torch.Tensor) -> torch.Tensor:
+    """``out[r] = gelu_tanh(gate[r]) * table[tokens[r], col : col + width]``: a gate on the numbers a token id brings."""
+    _gpu(gate, "gate")
+    _gpu(tokens, "tokens", torch.int32)
+    _gpu(table, "table", gate.dtype)
+    _gpu(out, "out", gate.dtype)
+    rows, width = gate.shape
+    if not (gate.stride(1) == 1 and out.shape == gate.shape and out.is_contiguous() and tokens.numel() >= rows and
+            tokens.is_contiguous()):
+        raise KernelError("token_gate: gate [rows, width] with unit column stride, out contiguous, a token id a row")
+    if not (table.dim() == 2 and table.stride(1) == 1 and 0 <= col and col + width <= table.shape[1]):
+        raise KernelError("token_gate: the run of columns lies outside the table")
+    _check(_fn("activation", "dryft_token_gate")(_ptr(gate), gate.stride(0), _ptr(tokens), _ptr(table), table.stride(0),
+                                                 int(col), table.shape[0], _ptr(out), rows, width,
+                                                 _float_flag(gate, "gate"), _stream()), "token_gate")
+    return out
+
+
+def blend_columns(a: torch.Tensor, b: torch.Tensor, lam: torch.Tensor) -> torch.Tensor:
+    """``a <- (1 - lam) a + lam b`` in place; ``a`` and ``b`` are ``[rows, width]`` column runs of wider tensors,
+    ``lam`` one float32 on the device."""
+    _gpu(a, "a")
+    _gpu(b, "b", a.dtype)
+    _gpu(lam, "lam", torch.float32)
+    if not (a.dim() == 2 and a.shape == b.shape and a.stride(1) == 1 and b.stride(1) == 1 and lam.numel() == 1):
+        raise KernelError("blend_columns: a and b [rows, width] with unit column stride, lam one number")
+    _check(_fn("activation", "dryft_blend_columns")(_ptr(a), a.stride(0), _ptr(b), b.stride(0), _ptr(lam), a.shape[0],
+                                                    a.shape[1], _float_flag(a, "a"), _stream()), "blend_columns")
+    return a
+
+
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _gpu(gate_up, "gate_up")
     _gpu(out, "out", gate_up.dtype)
@@ -479,10 +525,12 @@ def _check_pages(k_pages, v_pages, page_table, n_kv: int, head_dim: int, dtype, 
 # --------------------------------------------------------------------------------------- attention
 def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: int, n_kv: int, head_dim: int,
               scale: float, window: int, *, v_dim: int | None = None, softcap: float = 0.0, sink=None,
-              exact_p: bool = False) -> None:
+              exact_p: bool = False, chunk: int = 0, rel=None) -> None:
     """``v_dim``: the values' width where it differs from the keys'; ``softcap`` > 0: scores become
     ``cap * tanh(s / cap)``; ``sink``: float32 ``[heads]`` whose exp() joins each head's denominator; ``exact_p``:
-    the probabilities weigh the values unrounded."""
+    the probabilities weigh the values unrounded; ``chunk`` > 0: a row sees the keys of its own run of so many
+    positions instead of a window; ``rel``: float32 ``[distances, heads]``, a bias by distance added to the scaled
+    score (the last row serves every larger distance)."""
     _gpu(q, "q")
     is_f32 = _float_flag(q, "q")
     v_dim = head_dim if v_dim is None else int(v_dim)
@@ -503,10 +551,19 @@ def attn_rows(q, k_pages, v_pages, page_table, row_slot, row_pos, out, n_heads: 
             raise KernelError(f"{name}: needs {rows} entries")
     if not (n_heads <= 65535):
         raise KernelError("attn_rows: too many heads")
+    _check_rel(rel, n_heads)
     _check(_fn("attn_rows", "dryft_attn_rows")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(row_slot), _ptr(row_pos),
         _ptr(out), rows, n_heads, n_kv, head_dim, v_dim, float(scale), int(window), float(softcap), _ptr(sink),
-        int(bool(exact_p)), is_f32, _stream()), "attn_rows")
+        int(bool(exact_p)), int(chunk), _ptr(rel), rel.shape[0] if rel is not None else 0, is_f32, _stream()),
+        "attn_rows")
+
+
+def _check_rel(rel, n_heads: int) -> None:
+    if rel is not None:
+        _gpu(rel, "rel", torch.float32)
+        if not (rel.dim() == 2 and rel.shape[1] == n_heads and rel.shape[0] >= 1 and rel.is_contiguous()):
+            raise KernelError(f"rel: needs contiguous float32 [distances, {n_heads}]")
 
 
 def _check_sink(sink, n_heads: int) -> None:
@@ -1520,11 +1577,12 @@ def rms_segments(src, col: int, w_a, out_a, n_a: int, w_b, out_b, eps: float) ->
 
 
 def latent_rope_kv(q_raw, kv, down, krot_col: int, cos, sin, rot: int, row_slot, row_pos, q_out, k_pages, v_pages,
-                   page_table, write_kv: bool, n_heads: int, plain: int, rot_dim: int, v_dim: int, page_dv: int) -> None:
+                   page_table, write_kv: bool, n_heads: int, plain: int, rot_dim: int, v_dim: int, page_dv: int,
+                   pairs: bool = False) -> None:
     """Queries ``[plain | rotated]`` per head from ``q_raw``; keys ``[that head's plain part of kv | the one rotated
     part at column krot_col of down]``; values from ``kv`` after the keys. The rotated parts' first ``rot`` features
-    turn, feature ``i`` with ``i + rot/2``, with float32 tables; keys and values go to their pages (values ``page_dv``
-    wide, of which ``v_dim`` are written)."""
+    turn, feature ``i`` with ``i + rot/2`` (with ``pairs``: feature ``2i`` with ``2i + 1``), with float32 tables; keys
+    and values go to their pages (values ``page_dv`` wide, of which ``v_dim`` are written)."""
     _gpu(q_raw, "q_raw")
     is_f32 = _float_flag(q_raw, "q_raw")
     rows, key_dim = q_raw.shape[0], plain + rot_dim
@@ -1557,12 +1615,14 @@ def latent_rope_kv(q_raw, kv, down, krot_col: int, cos, sin, rot: int, row_slot,
     _check(_fn("latent", "dryft_latent_rope_kv")(
         _ptr(q_raw), _ptr(kv), _ptr(down), down.stride(0), krot_col, _ptr(cos), _ptr(sin), rot, _ptr(row_slot),
         _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1],
-        int(bool(write_kv)), rows, n_heads, plain, rot_dim, v_dim, page_dv, is_f32, _stream()), "latent_rope_kv")
+        int(bool(write_kv)), rows, n_heads, plain, rot_dim, v_dim, page_dv, int(bool(pairs)), is_f32, _stream()),
+        "latent_rope_kv")
 
 
-def head_gate(attn, down, g_col: int, out, n_heads: int, v_dim: int) -> None:
+def head_gate(attn, down, g_col: int, out, n_heads: int, v_dim: int, per_element: bool = False) -> None:
     """``out[row, head, :] = attn[row, head, :v_dim] * sigmoid(down[row, g_col + head])``; ``attn``'s heads may be
-    wider than ``v_dim``, ``out`` is packed ``[rows, heads * v_dim]``."""
+    wider than ``v_dim``, ``out`` is packed ``[rows, heads * v_dim]``. With ``per_element`` every output has a gate
+    of its own, ``down[row, g_col + head * v_dim + j]``."""
     _gpu(attn, "attn")
     rows = down.shape[0]
     _gpu(down, "down", attn.dtype)
@@ -1572,10 +1632,11 @@ def head_gate(attn, down, g_col: int, out, n_heads: int, v_dim: int) -> None:
         raise KernelError("head_gate: attn must be contiguous [rows, heads, >= v_dim]")
     if not (out.shape == (rows, n_heads * v_dim) and out.is_contiguous()):
         raise KernelError("head_gate: out must be contiguous [rows, heads * v_dim]")
-    if not (down.stride(1) == 1 and 0 <= g_col and g_col + n_heads <= down.shape[1]):
+    if not (down.stride(1) == 1 and 0 <= g_col and g_col + n_heads * (v_dim if per_element else 1) <= down.shape[1]):
         raise KernelError("head_gate: the gates lie outside down's columns")
     _check(_fn("latent", "dryft_head_gate")(_ptr(attn), _ptr(down), down.stride(0), g_col, _ptr(out), rows, n_heads,
-                                            in_dim, v_dim, _float_flag(attn, "attn"), _stream()), "head_gate")
+                                            in_dim, v_dim, int(bool(per_element)), _float_flag(attn, "attn"), _stream()),
+           "head_gate")
 
 
 # ------------------------------------------------------------------------------------------ routed experts
@@ -1583,15 +1644,19 @@ MOE_MAX_EXPERTS = 512
 MOE_TILE = 64
 
 
-def moe_route(logits, correction, n_experts: int, groups: int, keep: int, scale: float, chosen, weights) -> None:
+def moe_route(logits, correction, n_experts: int, groups: int, keep: int, scale: float, chosen, weights, *,
+              softmax: bool = False, group_best: bool = False, renorm: bool = True) -> None:
     """Per row of float32 ``logits`` (their first ``n_experts`` columns): the ``top`` experts by ``sigmoid + correction``
     among the ``keep`` best of ``groups`` groups (a group's score: its two largest such scores), and their weights
-    ``sigmoid / (sum of the chosen sigmoids + 1e-20) * scale``. ``chosen`` int32 and ``weights`` float32 ``[rows, top]``."""
+    ``sigmoid / (sum of the chosen sigmoids + 1e-20) * scale``. ``chosen`` int32 and ``weights`` float32 ``[rows, top]``.
+    ``softmax``: scores are the softmax over all experts instead; ``correction`` None: none; ``group_best``: a group
+    scores as its best expert; ``renorm`` off: the weights are the scores times ``scale`` as they are."""
     _gpu(logits, "logits", torch.float32)
     rows, top = chosen.shape
     if not (logits.dim() == 2 and logits.shape[0] == rows and logits.stride(1) == 1 and logits.shape[1] >= n_experts):
         raise KernelError("moe_route: logits must be float32 [rows, >= experts] with unit column stride")
-    _f32_vector(correction, "correction", n_experts)
+    if correction is not None:
+        _f32_vector(correction, "correction", n_experts)
     _gpu(chosen, "chosen", torch.int32)
     _gpu(weights, "weights", torch.float32)
     if not (chosen.is_contiguous() and weights.shape == (rows, top) and weights.is_contiguous()):
@@ -1600,7 +1665,8 @@ def moe_route(logits, correction, n_experts: int, groups: int, keep: int, scale:
             keep * (n_experts // groups) >= top):
         raise KernelError("moe_route: sizes the router does not take")
     _check(_fn("moe", "dryft_moe_route")(_ptr(logits), logits.stride(0), _ptr(correction), n_experts, groups, keep, top,
-                                         float(scale), _ptr(chosen), _ptr(weights), rows, _stream()), "moe_route")
+                                         float(scale), _ptr(chosen), _ptr(weights), rows, int(bool(softmax)),
+                                         int(bool(group_best)), int(bool(renorm)), _stream()), "moe_route")
 
 
 class MoePlan:
@@ -1645,13 +1711,15 @@ def moe_table_route(tokens, table, n_experts: int, chosen, weights) -> None:
                                                table.shape[0], n_experts, _stream()), "moe_table_route")
 
 
-def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple | None = None) -> None:
+def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple | None = None, act: str | None = None) -> None:
     """``out[place] = W_e a_row`` for every place of the plan, ``e`` the place's expert. ``top`` > 0: ``a`` is
     ``[rows, K]`` and a place's operand is row ``pair // top``; ``top`` == 0: ``a`` is ``[pairs, K]`` in place order.
     ``w`` is ``[experts, N, K]``; with ``glu = (limit, alpha)`` it holds gate rows then up rows (``N = 2 I``) and
     ``out [pairs, I]`` receives the clamped gated unit of the two, ``g sigmoid(alpha g) (u + 1)``; ``glu = (limit, alpha,
     offset)`` puts ``offset`` in the place of that 1 (``(inf, 1, 0)`` is ``silu(gate) * up``). ``out`` may be float32
-    for a plain product."""
+    for a plain product. ``act="relu2"`` (no gate): ``out`` receives the square of relu of the product."""
+    if act not in (None, "relu2") or (act and glu):
+        raise KernelError("moe_products: act is None or 'relu2', and goes without a gate")
     _gpu(a, "a")
     _gpu(w, "w", a.dtype)
     _gpu(out, "out")
@@ -1671,7 +1739,7 @@ def moe_products(a, w, plan: MoePlan, out, top: int, glu: tuple | None = None) -
     _check(_fn("moe", "dryft_moe_product")(
         _ptr(a), a.stride(0), _ptr(w), _ptr(plan.sorted_pair), _ptr(plan.tiles[0]), _ptr(plan.tiles[1]),
         _ptr(plan.tiles[2]), _ptr(plan.n_tiles), plan.max_tiles, _ptr(out), 1 if out.dtype == torch.float32 else 0,
-        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), float(offset), plan.most_places,
+        int(top), n_out, k, 1 if glu else 0, float(limit), float(alpha), float(offset), 1 if act else 0, plan.most_places,
         _float_flag(a, "a"), _stream()),
         "moe_products")
 

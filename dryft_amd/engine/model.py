@@ -148,6 +148,7 @@ class DecoderModel:
         stream as that run leaves it (float32, everything pending added): a way to look, not part of the step."""
         ctx.positions = self.positions
         ctx.tokens = tokens
+        ctx.shared.clear()
         x = self.embedding.forward(tokens)
         ctx.embedded = x
         pending = None

@@ -77,3 +77,4 @@ from . import qwen3 as _qwen3  # noqa: E402,F401  (registers Qwen3ForCausalLM)
 from . import piralix as _piralix  # noqa: E402,F401  (registers Piralix)
 from . import fetedra as _fetedra  # noqa: E402,F401  (registers Fetedra)
 from . import barilix as _barilix  # noqa: E402,F401  (registers Barilix)
+from . import podenex as _podenex  # noqa: E402,F401  (registers Podenex)

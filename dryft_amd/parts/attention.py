@@ -15,7 +15,15 @@ the output projection (tensor ``g_proj``, fused into the q/k/v product); attenti
 every channel of q, k and v right after the projection (``conv_taps``; the last ``taps - 1`` projected values of a
 sequence are then part of its state, beside its keys and values); and a position encoding with float tables, over
 neighbouring pairs (``PairRotaryPositions``) or over halves (``HalfRotaryPositions``; this one also after the per-head
-norms, in float). Any of these takes the step down ``_forward_general``.
+norms, in float); a sink of a fixed score instead of a learned one (``sink_value``: 0 puts ``1`` beside the sum of
+the exponentials); chunks instead of a window (``chunk``: a row sees the earlier keys of its own run of so many
+positions, runs counted from position 0); a learned bias by distance added to the scaled score (``distance_bias =
+(rows, far)``, tensor ``rel [rows, heads]``: distances below ``rows / 2`` have a row each, the others share the upper
+half on a logarithmic scale that reaches the last row at ``far``); one output gate per head instead of one per
+feature (``output_gate="head"``); and values that lean on those of an earlier layer (``value_mix = (name, first)``:
+the first layer of that name leaves its values of the step's rows in the step context, every later one takes ``(1 -
+l) v + l v_first`` with its own learned ``l``, tensor ``vmix``, before anything is cached). Any of these takes the
+step down ``_forward_general``.
 
 The part knows nothing of the model around it: sizes and constants are constructor arguments, the
 position encoding is looked up by name in the step context, and its storage is the cache line it
@@ -54,12 +62,23 @@ def add_bias(delta, bias: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def distance_row(n: int, rows: int, far: int) -> int:
+    """The row of a bias table that distance ``n`` reads: its own below half the table, then
+    ``half + floor(log(n / half) / log(far / half) * (rows - half))``, at most the last."""
+    half = rows // 2
+    if n < half:
+        return n
+    return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half))))
+
+
 class GQAAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: float | None = None, positions: str | None = None, rotary_dim: int | None = None,
                  window: int | None = None, scale: float | None = None, value_dim: int | None = None,
-                 softcap: float | None = None, sink: bool = False, output_gate: bool = False,
-                 float_weights: bool = False, bias: bool = False, conv_taps: int | None = None):
+                 softcap: float | None = None, sink: bool = False, output_gate: bool | str = False,
+                 float_weights: bool = False, bias: bool = False, conv_taps: int | None = None,
+                 sink_value: float | None = None, chunk: int | None = None,
+                 distance_bias: tuple[int, int] | None = None, value_mix: tuple[str, bool] | None = None):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} kv heads evenly")
         if not 0 < head_dim <= MAX_HEAD_DIM:
@@ -76,17 +95,33 @@ class GQAAttention(Mixer):
         if not 0 < self.value_dim <= MAX_HEAD_DIM:
             raise ValueError(f"value_dim must lie in 1..{MAX_HEAD_DIM}, got {value_dim}")
         self.softcap = float(softcap) if softcap else 0.0
+        if output_gate not in (False, True, "head"):
+            raise ValueError(f"output_gate is False, True (a gate per feature) or 'head', got {output_gate!r}")
         self.has_sink, self.output_gate, self.float_weights = bool(sink), bool(output_gate), bool(float_weights)
+        self.head_gate = output_gate == "head"
+        self.sink_value = None if sink_value is None else float(sink_value)
+        if self.has_sink and self.sink_value is not None:
+            raise ValueError("a sink is learned (sink) or fixed (sink_value), not both")
+        self.chunk = int(chunk) if chunk else None
+        if self.chunk and self.window:
+            raise ValueError("a mixer has a window or chunks, not both")
+        self.distance_bias = (int(distance_bias[0]), int(distance_bias[1])) if distance_bias else None
+        if self.distance_bias and not (self.distance_bias[0] == -1 or 2 <= self.distance_bias[0] < 2 * self.distance_bias[1]):
+            raise ValueError(f"a bias by distance needs at least 2 rows (-1: as many as the checkpoint holds) and a far "
+                             f"distance beyond half of them, got {self.distance_bias}")
+        self.value_mix = (str(value_mix[0]), bool(value_mix[1])) if value_mix else None
         self.q_dim, self.kv_dim = self.n_heads * self.head_dim, self.n_kv * self.head_dim
         self.v_dim, self.o_dim = self.n_kv * self.value_dim, self.n_heads * self.value_dim
         self.has_bias, self.conv_taps = bool(bias), int(conv_taps) if conv_taps else 0
         if self.conv_taps > ops.CONV_MAX_TAPS:
             raise ValueError(f"the convolution takes at most {ops.CONV_MAX_TAPS} taps, got {conv_taps}")
+        self.g_dim = (self.n_heads if self.head_gate else self.o_dim) if self.output_gate else 0
         self.extended = bool(self.value_dim != self.head_dim or self.softcap or self.has_sink or self.output_gate or
-                             self.float_weights or self.has_bias or self.conv_taps)
+                             self.float_weights or self.has_bias or self.conv_taps or self.sink_value is not None or
+                             self.chunk or self.distance_bias or self.value_mix)
         self.conv_channels = self.q_dim + self.kv_dim + self.v_dim
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.sink = None
-        self.in_bias = self.o_bias = self.conv_w = self.conv_wt = None
+        self.in_bias = self.o_bias = self.conv_w = self.conv_wt = self.rel = self.vmix = None
 
     def tensor_specs(self):
         specs = {"q_proj": matrix((self.q_dim, self.hidden)), "k_proj": matrix((self.kv_dim, self.hidden)),
@@ -94,7 +129,11 @@ class GQAAttention(Mixer):
         if self.has_sink:
             specs["sink"] = ((self.n_heads,), VECTOR, "normal")
         if self.output_gate:
-            specs["g_proj"] = matrix((self.o_dim, self.hidden))
+            specs["g_proj"] = matrix((self.g_dim, self.hidden))
+        if self.distance_bias:
+            specs["rel"] = ((self.distance_bias[0], self.n_heads), VECTOR, "normal")
+        if self.value_mix:
+            specs["vmix"] = ((), VECTOR, "normal")
         if self.qk_norm_eps is not None:
             specs["q_norm"] = ((self.head_dim,), VECTOR, "ones")
             specs["k_norm"] = ((self.head_dim,), VECTOR, "ones")
@@ -111,6 +150,17 @@ class GQAAttention(Mixer):
         self.w_qkv = torch.cat(fused, dim=0).contiguous()
         if self.has_sink:
             self.sink = tensors["sink"].float().contiguous()
+        elif self.sink_value is not None:
+            self.sink = torch.full((self.n_heads,), self.sink_value, dtype=torch.float32, device=self.w_qkv.device)
+        if self.distance_bias:
+            # a row per distance 0..far, so that the kernels look a bias up without logarithms
+            rows, far = tensors["rel"].shape[0], self.distance_bias[1]
+            if not 2 <= rows < 2 * far:
+                raise ValueError(f"a bias table of {rows} rows does not go with a far distance of {far}")
+            index = torch.tensor([distance_row(n, rows, far) for n in range(far + 1)], device=self.w_qkv.device)
+            self.rel = tensors["rel"].float()[index].contiguous()
+        if self.value_mix:
+            self.vmix = tensors["vmix"].float().reshape(1).contiguous()
         self.w_o = tensors["o_proj"]
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = tensors["q_norm"], tensors["k_norm"]
@@ -127,14 +177,17 @@ class GQAAttention(Mixer):
             self.conv_wt = self.conv_w.t().contiguous()                  # tap by tap, for 8 channels a thread
 
     def cache_need(self):
-        kv = KVNeed(self.n_kv, self.head_dim, self.window, self.value_dim if self.value_dim != self.head_dim else None)
+        # a row of a chunked mixer never looks further back than a chunk: the pages behind that are given back
+        kv = KVNeed(self.n_kv, self.head_dim, self.window or self.chunk,
+                    self.value_dim if self.value_dim != self.head_dim else None)
         if self.conv_taps > 1:
             return {"kv": kv, "tail": conv_need(self.conv_taps, self.conv_channels)}
         return kv
 
     def kernel_modules(self, dtype):
         return ("gemm", "rope_kv", "attn_rows") + (("attn_mfma",) if dtype == torch.bfloat16 else ()) + \
-            (("activation",) if self.output_gate else ()) + (("conv", "norm") if self.conv_taps or self.has_bias else ())
+            (("activation",) if self.output_gate or self.value_mix else ()) + (("latent",) if self.head_gate else ()) + \
+            (("conv", "norm") if self.conv_taps or self.has_bias else ())
 
     def _forward_general(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
         """Every option, in float arithmetic on the kernel that takes one (row, head) a workgroup. Returns the output
@@ -159,6 +212,16 @@ class GQAAttention(Mixer):
             # biases and the short convolution: q | k | v as one run of channels, each with its own history
             src = short_conv(proj, 0, self.conv_channels, self.conv_w, ctx, tail, writes_cache, in_bias=self.in_bias,
                              weight_t=self.conv_wt)
+        if self.value_mix:
+            name, first = self.value_mix
+            v_cols = src[:, self.q_dim + self.kv_dim:self.q_dim + self.kv_dim + self.v_dim]
+            if first:
+                ctx.shared["values:" + name] = v_cols
+            else:
+                earlier = ctx.shared.get("values:" + name)
+                if earlier is None or earlier.shape != v_cols.shape:
+                    raise ValueError(f"values {name!r}: no earlier layer of this step has left values of this shape")
+                ops.blend_columns(v_cols, earlier, self.vmix)
         q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
         if isinstance(table, PairRotaryPositions):
             if self.qk_norm_eps is not None:
@@ -171,7 +234,8 @@ class GQAAttention(Mixer):
                                   line.page_table, writes_cache, H, G, D, Dv)
         # bfloat16 on the matrix cores where they take the sizes (keys and values of one width, a multiple of 16);
         # float32, and the other sizes, on the kernel that takes one (row, head) a workgroup in float arithmetic
-        matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0
+        matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0 and \
+            not self.chunk and self.rel is None
         window = self.window or 0
         if matrix_cores and ctx.max_q_len == 1:
             out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
@@ -192,12 +256,17 @@ class GQAAttention(Mixer):
         else:
             out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, G, D, self.scale,
-                          window, v_dim=Dv, softcap=self.softcap, sink=self.sink, exact_p=self.float_weights)
+                          window, v_dim=Dv, softcap=self.softcap, sink=self.sink, exact_p=self.float_weights,
+                          chunk=self.chunk or 0, rel=self.rel)
         out = out.view(rows, self.o_dim)
         if self.output_gate:
             gated = torch.empty_like(out)
             g_col = self.q_dim + self.kv_dim + self.v_dim
-            out = ops.sigmoid_gate(out, proj[:, g_col:g_col + self.o_dim], gated)
+            if self.head_gate:
+                ops.head_gate(out, proj, g_col, gated, H, Dv)
+                out = gated
+            else:
+                out = ops.sigmoid_gate(out, proj[:, g_col:g_col + self.o_dim], gated)
         return linear(out, self.w_o, allow_partials=True)
 
     def forward_split(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
@@ -303,6 +372,8 @@ class GQAAttention(Mixer):
             if self.window:
                 full = max(0, min(last, self.window) - first + 1)          # rows that still see every key
                 seen += (2 * first + full - 1) * full // 2 + (q - full) * self.window
+            elif self.chunk:
+                seen += sum(p % self.chunk + 1 for p in range(start, start + q))
             else:
                 seen += (first + last) * q // 2
         return super().flops(rows, spans) + 2.0 * (self.q_dim + self.o_dim) * seen
@@ -315,7 +386,7 @@ class GQAAttention(Mixer):
         """
         blocks = self.n_kv * ((self.n_heads // self.n_kv + 15) // 16)
         want = _RESIDENT_WORKGROUPS // (n_seqs * blocks)
-        span = self.window if self.window else max_kv_len
+        span = self.window or getattr(self, "chunk", None) or max_kv_len
         pages = max(1, (span + 63) // 64)
         return max(1, min(want, _MAX_SPLITS, pages))
 

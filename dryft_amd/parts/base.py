@@ -59,6 +59,9 @@ class StepContext:
     positions: dict[str, Any] = field(default_factory=dict)   # name -> position encoding, tables ready
     embedded: torch.Tensor | None = None    # the embedding's output of this step's rows, for parts that come back to it
     tokens: torch.Tensor | None = None      # the step's token ids (int32, a row each), for parts that look them up
+    # what a part of an earlier layer leaves for parts of later layers of the same step, by a name the plan gives
+    # both (the values a first attention layer computed, which later ones lean on); emptied when a step begins
+    shared: dict[str, Any] = field(default_factory=dict)
     _tiles: dict[int, tuple[torch.Tensor, int]] = field(default_factory=dict, repr=False)
     _kept: dict[Any, torch.Tensor] = field(default_factory=dict, repr=False)
 

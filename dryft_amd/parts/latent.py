@@ -13,6 +13,11 @@ and the attention kernels of the library read such pages (head widths up to 256,
 the width of a single shared head soon exceeds). Where the matrix cores serve the step (bfloat16, key width a
 multiple of 16) the values' pages are as wide as the keys', the columns beyond ``value_dim`` staying zero.
 
+Other forms, by constructor arguments: no sink (``sink=False``: an ordinary softmax); a gate per output feature
+instead of one per head (``gate="element"``: ``sigmoid(W_g h)`` is as wide as the concatenated heads); and, with a
+position encoding over neighbouring pairs (``PairRotaryPositions``), feature ``2i`` of the rotated part turns with
+feature ``2i + 1``.
+
 Float arithmetic in both precisions: both latent norms, the rotation with float32 tables, scores, softmax with its
 sink, the gate's sigmoid.
 """
@@ -30,11 +35,16 @@ from . import register_part
 from .attention import GQAAttention
 from .base import Mixer, StepContext, matrix
 from .linear import linear
+from .rope import PairRotaryPositions
 
 
 class LatentAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int, value_dim: int, q_rank: int,
-                 kv_rank: int, scale: float, norm_eps: float, positions: str | None = None, window: int | None = None):
+                 kv_rank: int, scale: float, norm_eps: float, positions: str | None = None, window: int | None = None,
+                 sink: bool = True, gate: str = "head"):
+        if gate not in ("head", "element"):
+            raise ValueError(f"gate is 'head' or 'element', got {gate!r}")
+        self.has_sink, self.element_gate = bool(sink), gate == "element"
         self.hidden, self.n_heads = int(hidden_size), int(num_heads)
         self.plain, self.rot_dim, self.value_dim = int(head_dim), int(rot_dim), int(value_dim)
         self.key_dim = self.plain + self.rot_dim
@@ -47,12 +57,15 @@ class LatentAttention(Mixer):
 
     def tensor_specs(self):
         H = self.n_heads
-        return {"q_down": matrix((self.q_rank, self.hidden)), "q_norm": ((self.q_rank,), VECTOR, "ones"),
+        specs = {"q_down": matrix((self.q_rank, self.hidden)), "q_norm": ((self.q_rank,), VECTOR, "ones"),
                 "q_up": matrix((H * self.key_dim, self.q_rank)),
                 "kv_down": matrix((self.kv_rank + self.rot_dim, self.hidden)), "kv_norm": ((self.kv_rank,), VECTOR, "ones"),
                 "k_up": matrix((H * self.plain, self.kv_rank)), "v_up": matrix((H * self.value_dim, self.kv_rank)),
-                "sink": ((H,), VECTOR, "normal"), "g_proj": matrix((H, self.hidden)),
+                "g_proj": matrix((H * self.value_dim if self.element_gate else H, self.hidden)),
                 "o_proj": matrix((self.hidden, H * self.value_dim))}
+        if self.has_sink:
+            specs["sink"] = ((H,), VECTOR, "normal")
+        return specs
 
     def load(self, tensors):
         # one product for everything that reads h: the queries' latent | the latent and the rotated key part | gates
@@ -61,7 +74,8 @@ class LatentAttention(Mixer):
         self.w_ukv = torch.cat([tensors["k_up"], tensors["v_up"]], dim=0).contiguous()
         self.w_o = tensors["o_proj"]
         self.q_norm, self.kv_norm = tensors["q_norm"].float().contiguous(), tensors["kv_norm"].float().contiguous()
-        self.sink = tensors["sink"].float().contiguous()
+        if self.has_sink:
+            self.sink = tensors["sink"].float().contiguous()
 
     def _matrix_cores(self) -> bool:
         return self.compute_dtype == torch.bfloat16 and self.key_dim % MATRIX_CORE_HEAD_STEP == 0 and \
@@ -80,12 +94,12 @@ class LatentAttention(Mixer):
     def forward(self, h: torch.Tensor, ctx: StepContext, line: KVLine, writes_cache: bool):
         rows, H, D, Dv = h.shape[0], self.n_heads, self.key_dim, self.value_dim
         cos = sin = None
-        rot = 0
+        rot, pairs = 0, False
         if self.positions:
             table = ctx.positions[self.positions]
             if ctx.max_kv_len > table.n_positions:
                 raise ValueError(f"position tables cover {table.n_positions} positions, the step reaches {ctx.max_kv_len}")
-            cos, sin, rot = table.cos, table.sin, table.dims
+            cos, sin, rot, pairs = table.cos, table.sin, table.dims, isinstance(table, PairRotaryPositions)
         down = linear(h, self.w_down)                               # c_q | c | rotated key part | gates
         c_q = torch.empty((rows, self.q_rank), dtype=h.dtype, device=h.device)
         c_kv = torch.empty((rows, self.kv_rank), dtype=h.dtype, device=h.device)
@@ -95,7 +109,8 @@ class LatentAttention(Mixer):
         q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
         page_dv = self._page_value_dim()
         ops.latent_rope_kv(q_raw, kv, down, self.q_rank + self.kv_rank, cos, sin, rot, ctx.row_slot, ctx.row_pos, q,
-                           line.k, line.v, line.page_table, writes_cache, H, self.plain, self.rot_dim, Dv, page_dv)
+                           line.k, line.v, line.page_table, writes_cache, H, self.plain, self.rot_dim, Dv, page_dv,
+                           pairs=pairs)
         window = self.window or 0
         if self._matrix_cores() and ctx.max_q_len == 1:
             out = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
@@ -116,7 +131,7 @@ class LatentAttention(Mixer):
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, H, D, self.scale,
                           window, v_dim=page_dv, sink=self.sink, exact_p=True)
         gated = torch.empty((rows, H * Dv), dtype=h.dtype, device=h.device)
-        ops.head_gate(out, down, self.q_rank + self.kv_rank + self.rot_dim, gated, H, Dv)
+        ops.head_gate(out, down, self.q_rank + self.kv_rank + self.rot_dim, gated, H, Dv, per_element=self.element_gate)
         return linear(gated, self.w_o, allow_partials=True)
 
     def decode_splits(self, n_seqs: int, max_kv_len: int) -> int:

@@ -75,5 +75,29 @@ class ClampedGLU(FeedForward):
         return linear(act, self.w_down, allow_partials=True)
 
 
+class SquaredReLU(FeedForward):
+    """``down( relu(up(h))^2 )``, dense, no gate, no bias."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden, self.inter = int(hidden_size), int(intermediate_size)
+        self.w_up: torch.Tensor | None = None
+        self.w_down: torch.Tensor | None = None
+
+    def tensor_specs(self):
+        return {"up_proj": matrix((self.inter, self.hidden)), "down_proj": matrix((self.hidden, self.inter))}
+
+    def load(self, tensors):
+        self.w_up, self.w_down = tensors["up_proj"], tensors["down_proj"]
+
+    def kernel_modules(self, dtype):
+        return ("gemm", "activation")
+
+    def forward(self, h, ctx):
+        act = torch.empty((h.shape[0], self.inter), dtype=h.dtype, device=h.device)
+        ops.relu_squared(linear(h, self.w_up), act)
+        return linear(act, self.w_down, allow_partials=True)
+
+
 register_part("swiglu", SwiGLU)
+register_part("squared_relu", SquaredReLU)
 register_part("clamped_glu", ClampedGLU)

@@ -12,6 +12,10 @@ due meanwhile, and norms the stream for its own first branch, in one launch.
 ``SandwichBlock``    mixer and feed-forward, each between two norms; ``SandwichMixerBlock`` has the mixer alone.
 ``PostNormBlock``    ``x <- x + norm(branch(x))``: the branches read the stream as it is, only their outputs are
                      normed; ``PostNormMixerBlock`` has the mixer alone.
+``PreNormBlock``     ``x <- x + branch(norm(x))``: a norm in front of every branch and none behind it; optionally a
+                     third sublayer (``TokenSide``) that reads the stream as it is.
+``TokenSide``        what a token id brings to a layer: a few numbers from a table, gated by the stream, projected
+                     to the width and rms-normed.
 ``PassEntry``        what a pass over a run of layers begins with: one learned vector per pass is added to the
                      stream, and from the second pass on the embedding's output once more.
 """
@@ -23,7 +27,8 @@ import torch
 from ..csrc import ops
 from ..weights.spec import VECTOR
 from . import register_block, register_part
-from .base import Deferred, FeedForward, Mixer, Norm, Partials, StepContext, StreamPart
+from .base import Deferred, FeedForward, Mixer, Norm, Part, Partials, StepContext, StreamPart, matrix
+from .linear import linear
 
 
 class StreamRMSNorm(Norm):
@@ -180,6 +185,83 @@ class PostNormMixerBlock(PostNormBlock):
     roles = ("mixer", "mixer_post_norm")
 
 
+class TokenSide(Part):
+    """A sublayer fed by the token id: ``e`` = columns ``[index * dim, (index + 1) * dim)`` of ``table[token]``,
+    ``g = gelu_tanh(W_gate x) * e``, ``y = W_proj g``, and what enters the stream is ``y / sqrt(mean(y^2) + eps) * w``
+    (an rms norm with a plain weight, whatever the model's own norm is). ``x`` is the stream as it is, not normed.
+    ``forward`` hands the output on unadded, with its norm, as every sublayer of a float32 stream does. The table is
+    one tensor for all layers (the plan gives every layer's part the same checkpoint name)."""
+
+    def __init__(self, hidden_size: int, dim: int, index: int, count: int, vocab_size: int, eps: float):
+        self.hidden, self.dim, self.index, self.count = int(hidden_size), int(dim), int(index), int(count)
+        self.vocab = int(vocab_size)
+        if not 0 <= self.index < self.count:
+            raise ValueError(f"run {index} of the table's {count}")
+        self.norm = StreamRMSNorm(hidden_size, eps)
+        self.table = self.w_gate = self.w_proj = None
+
+    def tensor_specs(self):
+        return {"table": matrix((self.vocab, self.count * self.dim)), "gate": matrix((self.dim, self.hidden)),
+                "proj": matrix((self.hidden, self.dim)), "norm": ((self.hidden,), VECTOR, "ones")}
+
+    def load(self, tensors):
+        self.table, self.w_gate, self.w_proj = tensors["table"], tensors["gate"], tensors["proj"]
+        self.norm.compute_dtype = self.compute_dtype
+        self.norm.load({"weight": tensors["norm"]})
+
+    def kernel_modules(self, dtype):
+        return ("gemm", "activation", "norm")
+
+    def flops(self, rows, spans):
+        return 4.0 * rows * self.dim * self.hidden
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> Deferred:
+        gate = linear(x, self.w_gate)
+        g = torch.empty_like(gate)
+        ops.token_gate(gate, ctx.tokens, self.table, self.index * self.dim, g)
+        return Deferred(delta=linear(g, self.w_proj, allow_partials=True), norm=self.norm)
+
+
+class PreNormBlock:
+    """``x <- x + mixer(norm_a(x))``, then ``x <- x + ffn(norm_b(x))``, then (with a ``side``) ``x <- x + side(x)``.
+    The stream is float32 from the first sum on; a sublayer's output is handed on unadded and enters the stream in
+    the launch that norms it for the next reader. A mixer's output bias rides along as the vector of that sum."""
+
+    roles = ("mixer_norm", "mixer", "ffn_norm", "ffn")
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm | None = None, ffn: FeedForward | None = None,
+                 side: TokenSide | None = None):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.side = mixer_norm, mixer, ffn_norm, ffn, side
+
+    def parts(self):
+        return {role: getattr(self, role) for role in self.roles}
+
+    def forward(self, x, pending, ctx: StepContext, line, writes_cache: bool):
+        # the embedding's output starts the stream and other parts may read it again: never updated in place
+        x, h = self.mixer_norm.add_forward(x, pending, ctx.dtype, in_place=x is not ctx.embedded)
+        delta, bias = self.mixer.forward_split(h, ctx, line, writes_cache)
+        pending = Deferred(delta=delta, vector=bias)
+        if self.ffn is not None:
+            x, h = self.ffn_norm.add_forward(x, pending, ctx.dtype)
+            pending = Deferred(delta=self.ffn.forward(h, ctx))
+        if self.side is not None:
+            x, h = read_plain(x, pending, ctx.dtype)
+            pending = self.side.forward(h, ctx)
+        return x, pending
+
+
+class PreNormMixerBlock(PreNormBlock):
+    roles = ("mixer_norm", "mixer")
+
+
+class PreNormSideBlock(PreNormBlock):
+    roles = ("mixer_norm", "mixer", "ffn_norm", "ffn", "side")
+
+
+class PreNormMixerSideBlock(PreNormBlock):
+    roles = ("mixer_norm", "mixer", "side")
+
+
 class PassEntry(StreamPart):
     """``steps [passes, width]``: pass ``t`` begins by adding ``steps[t]`` to every row of the stream, and every pass
     but the first (when ``readd_embedding``) by adding the embedding's output of the row once more."""
@@ -213,6 +295,11 @@ class PassEntry(StreamPart):
 register_part("stream_rmsnorm", StreamRMSNorm)
 register_part("stream_layernorm", StreamLayerNorm)
 register_part("pass_entry", PassEntry)
+register_part("token_side", TokenSide)
+register_block("pre_norm", PreNormBlock)
+register_block("pre_norm_mixer", PreNormMixerBlock)
+register_block("pre_norm_side", PreNormSideBlock)
+register_block("pre_norm_mixer_side", PreNormMixerSideBlock)
 register_block("sandwich", SandwichBlock)
 register_block("sandwich_mixer", SandwichMixerBlock)
 register_block("post_norm", PostNormBlock)
