@@ -94,8 +94,9 @@ def weigh(scores, mask, values, group, sink=False):
 
 
 def mix_values(v, lam, v_first):
-    """Values of a later layer lean on those the first such layer computed for the same token."""
-    return (1 - lam) * v + lam * v_first
+    """Values of a later layer lean on those the first such layer computed for the same token (a token's values
+    taken as one vector over all its key/value heads)."""
+    return (1 - lam) * v + lam * v_first.reshape(v.shape)
 
 
 # ------------------------------------------------------------------------------------------ mixer 'attention'
