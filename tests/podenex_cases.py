@@ -1,7 +1,7 @@
 """Small Podenex configurations with weights of the tests' own making.
 
 The weights are drawn here, not by the library: matrices ``N(0, 1 / in)`` so that activations stay of order one, norm
-weights around one, convolution taps of order one, bias tables of order one, blends of values between 0.2 and 0.8,
+weights around one, convolution taps that keep a channel's size, bias tables of order one, blends of values between 0.2 and 0.8,
 everything rounded to bfloat16 so that both precisions read the same numbers.
 """
 
@@ -122,19 +122,19 @@ def tensors_for(cfg: dict, seed: int) -> dict[str, torch.Tensor]:
         if layer["type"] == "latent_attention":
             H, D, R, Dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
             mat(p + "mix.dq", m["q_rank"], W, 2.0); vec(p + "mix.dq.norm", m["q_rank"], 1.0, 0.3)
-            mat(p + "mix.uq", H * (D + R), m["q_rank"], 2.0)
+            mat(p + "mix.uq", H * (D + R), m["q_rank"], 1.4)
             mat(p + "mix.dkv", m["kv_rank"] + R, W, 2.0); vec(p + "mix.dkv.norm", m["kv_rank"], 1.0, 0.3)
-            mat(p + "mix.uk", H * D, m["kv_rank"], 2.0); mat(p + "mix.uv", H * Dv, m["kv_rank"], 2.0)
+            mat(p + "mix.uk", H * D, m["kv_rank"], 1.4); mat(p + "mix.uv", H * Dv, m["kv_rank"], 2.0)
             mat(p + "mix.g", H * Dv, W, 2.0); mat(p + "mix.o", W, H * Dv)
         else:
             H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
             for n, width in (("q", H * D), ("k", G * D), ("v", G * Dv)):
-                mat(p + "mix." + n, width, W, 2.0)
+                mat(p + "mix." + n, width, W, 2.0 if n == "v" else 1.4)
                 if layer["type"] == "attention_2":
                     vec(p + f"mix.{n}.b", width, 0.0, 0.5)
                 elif m.get("conv"):
                     taps = m["conv"]
-                    out[p + f"mix.{n}.conv"] = torch.randn(width, taps, generator=g) * (0.8 if taps > 1 else 1.0) + (0.5 if taps == 1 else 0.0)
+                    out[p + f"mix.{n}.conv"] = torch.randn(width, taps, generator=g) / taps ** 0.5 + (0.5 if taps == 1 else 0.0)
             mat(p + "mix.o", W, H * Dv)
             if layer["type"] == "attention_2":
                 vec(p + "mix.q.norm", D, 1.0, 0.3); vec(p + "mix.k.norm", D, 1.0, 0.3); vec(p + "mix.o.b", W, 0.0, 0.3)
