@@ -43,17 +43,36 @@ __device__ __forceinline__ float fast_tanh(float x) {
 
 // Options of the score that some designs use. A cap: s <- cap * tanh(s * scale / cap) (`pre` = scale / cap; 0: none).
 // A sink: one float per query head whose exp() joins the softmax's denominator and nothing else (null: none).
+// Chunks: a row sees the earlier keys of its own run of `chunk` positions, runs counted from position 0 (0: none;
+// a window then, or everything). A bias by distance: rel[min(pos - j, n_dist - 1)][head] (float, [n_dist][heads])
+// is added to the scaled score (null: none).
 struct ScoreCap {
   float cap = 0.f, pre = 0.f;
+  const float* rel = nullptr;          // the bias table at the column of the lane's (or unit's) head
+  int rel_stride = 0, n_dist = 0;
+  float rel_scale = 0.f;
 };
 struct ScoreOptions {
   float softcap;
   const float* sink;
+  int chunk;
+  const float* rel;
+  int n_dist;
 };
-__device__ __forceinline__ ScoreCap score_cap(const ScoreOptions& o, float scale) {
+__device__ __forceinline__ ScoreCap score_cap(const ScoreOptions& o, float scale, int n_heads = 0) {
   ScoreCap c;
   if (o.softcap > 0.f) { c.cap = o.softcap; c.pre = scale / o.softcap; }
+  if (o.rel != nullptr) { c.rel = o.rel; c.rel_stride = n_heads; c.n_dist = o.n_dist; c.rel_scale = scale; }
   return c;
+}
+// the same for one head
+__device__ __forceinline__ ScoreCap for_head(ScoreCap c, int head) {
+  if (c.rel != nullptr) c.rel += head;
+  return c;
+}
+// The first key a row at position `pos` sees.
+__device__ __forceinline__ int first_seen(int pos, int window, int chunk) {
+  return chunk > 0 ? pos - pos % chunk : (window > 0 ? max(0, pos - window + 1) : 0);
 }
 // 2^(sink in units of log2 e - m): what the sink adds to a row's sum whose reference maximum is m
 __device__ __forceinline__ float sink_term(const float* sink, int head, float m) {
@@ -161,6 +180,15 @@ __device__ __forceinline__ float page_softmax(RowBlock<KB>& st, f32x4 (&s)[4], b
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) s[t][i] = cap.cap * fast_tanh(s[t][i] * cap.pre);
+  }
+  if (cap.rel != nullptr) {                                   // s <- s * scale + bias[distance]; scale_log2 is log2(e) then
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int dist = min(max(hi_row - (key0 + 16 * t + 4 * g + i), 0), cap.n_dist - 1);   // hidden keys: any row
+        s[t][i] = fmaf(s[t][i], cap.rel_scale, cap.rel[(int64_t)dist * cap.rel_stride]);
+      }
   }
   float lane_max = -INFINITY;
 #pragma unroll
@@ -366,7 +394,8 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
     bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window, ScoreOptions opt) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   constexpr int U = GP * RP, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP;
-  const ScoreCap cap = score_cap(opt, scale);
+  const ScoreCap cap = score_cap(opt, scale, n_heads);
+  const int chunk = opt.chunk;
   // Two heads per wave: a workgroup takes one tile from each end of the list (grid: pairs of tiles x heads / 2).
   // Otherwise: one tile per workgroup, the ones with the most pages first, heads fastest (grid: heads x tiles),
   // so that the short tiles fill the compute units that the long ones leave.
@@ -406,18 +435,18 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
     row[rt] = (int64_t)cu_rows[seq] + first + c;
     pos0[rt] = pos_wave + 16 * rt;
     pos_row[rt] = row_valid[rt] ? pos0[rt] + c : -1;          // an absent row sees nothing
-    lo_row[rt] = window > 0 ? max(0, pos_row[rt] - window + 1) : 0;
+    lo_row[rt] = first_seen(pos_row[rt], window, chunk);
   }
   const int kvh = head0 / (n_heads / n_kv);
   RowBlock<KB> st[U];                                         // unit u: head u % GP, rows of tile u / GP
 #pragma unroll
   for (int u = 0; u < U; ++u)
     init_rows<KB>(st[u], q + (row[u / GP] * n_heads + head0 + u % GP) * head_dim, row_valid[u / GP], head_dim);
-  const int lo_wave = window > 0 ? max(0, pos_wave - window + 1) : 0;
+  const int lo_wave = first_seen(pos_wave, window, chunk);
   const int hi_wave = pos_wave + wave_rows - 1;               // below lo_wave for a wave without rows
-  const int lo_tile = window > 0 ? max(0, pos_tile - window + 1) : 0;
+  const int lo_tile = first_seen(pos_tile, window, chunk);
   const int hi_tile = pos_tile + min(TILE_ROWS, q_len - tile_first) - 1;
-  const float scale_log2 = (cap.cap > 0.f ? 1.f : scale) * 1.44269504088896340736f;
+  const float scale_log2 = (cap.cap > 0.f || cap.rel != nullptr ? 1.f : scale) * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   const int* table = page_table + (int64_t)slot * max_pages;
   const int pg_first = lo_tile / PAGE_TOKENS, pg_last = hi_tile / PAGE_TOKENS;
@@ -470,10 +499,12 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
         const int rt = u / GP;
         // every key of the page is seen by every row of the tile unless the page reaches past the tile's first
         // row, starts before a window's edge, or the tile has fewer than 16 rows
+        // or a chunk's start
         const bool masked = key0 + PAGE_TOKENS - 1 > pos0[rt] || rows[rt] < 16 ||
-                            (window > 0 && key0 < pos0[rt] + 15 - window + 1);
-        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], cap)
-                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], cap);
+                            key0 < first_seen(pos0[rt] + 15, window, chunk);
+        const ScoreCap mine = for_head(cap, head0 + u % GP);
+        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], mine)
+                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], mine);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
@@ -896,7 +927,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     const int* __restrict__ cu_rows, const int* __restrict__ kv_len, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_heads, int n_kv, int head_dim, float scale, int window, int n_splits,
     FusedQKV fused, bf16_t* k_pages_w, bf16_t* v_pages_w, bf16_t* __restrict__ out, ScoreOptions opt) {
-  const ScoreCap cap = score_cap(opt, scale);
+  ScoreCap cap = score_cap(opt, scale, n_heads);
   __shared__ float merge_o[SPLIT_WAVES][16][32 * KB + 1];
   __shared__ float merge_ml[SPLIT_WAVES][16][2];
   __shared__ __attribute__((aligned(16))) bf16_t q_lds[16][32 * KB];
@@ -914,7 +945,7 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
   const int* table = page_table + (int64_t)max(slot, 0) * max_pages;
   if (slot >= 0) {
     pos = kv_len[seq] - 1;                                     // the row's own position
-    lo = window > 0 ? max(0, pos - window + 1) : 0;
+    lo = first_seen(pos, window, opt.chunk);
     const int pg_lo = lo / PAGE_TOKENS;
     pg_hi = pos / PAGE_TOKENS;
     const int per = (pg_hi - pg_lo + n_splits) / n_splits;     // ceil(pages / splits)
@@ -922,7 +953,8 @@ __global__ __launch_bounds__(64 * SPLIT_WAVES, 2) void attn_split_kernel(
     pg_first = pg_lo + split * per;
     pg = pg_first + wave;
   }
-  const float scale_log2 = (cap.cap > 0.f ? 1.f : scale) * 1.44269504088896340736f;
+  const float scale_log2 = (cap.cap > 0.f || cap.rel != nullptr ? 1.f : scale) * 1.44269504088896340736f;
+  cap = for_head(cap, min(head, n_heads - 1));                 // a lane's row is a head here; absent rows read a valid column
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   PageK<KB> kf;
   PageV<KB> vf;
@@ -1207,9 +1239,9 @@ static int causal_entry(const void* q, const void* k_pages, const void* v_pages,
   const bool staged = mode == 5 || mode == 7;
   if (staged) mode -= 4;
   if (mode < 0 || mode > 3 || (mode == 2 && (group % 2 || head_dim > 128)) || (mode == 3 && head_dim > 128)) return -1;
-  // (the kernel that brings pages straight into LDS knows neither a cap nor a sink)
+  // (the kernel that brings pages straight into LDS knows neither a cap nor a sink, chunks or a bias)
   const bool direct_ok = head_dim == DIRECT_D && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0 &&
-                         !(opt.softcap > 0.f) && opt.sink == nullptr;
+                         !(opt.softcap > 0.f) && opt.sink == nullptr && opt.chunk == 0 && opt.rel == nullptr;
   if (mode == 0) {
     // Two units per wave (twice the rows of one head, or two heads of a kv group) use every piece of a page that
     // is read from LDS twice; they also halve the number of workgroups, so they need four of them for every
@@ -1245,11 +1277,12 @@ DRYFT_API int dryft_attn_causal_bf16(const void* q, const void* k_pages, const v
                                      int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                      const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads,
                                      int n_kv, int head_dim, float scale, int window, int mode, float softcap,
-                                     const float* sink, hipStream_t stream) {
+                                     const float* sink, int chunk, const float* rel, int n_dist, hipStream_t stream) {
   ProjectedQ none = {};
+  if (chunk < 0 || (chunk > 0 && window > 0) || (rel != nullptr && n_dist <= 0)) return -1;
   return causal_entry(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
                       max_tiles, out, n_heads, n_kv, head_dim, scale, window, mode, none, stream,
-                      ScoreOptions{softcap, sink});
+                      ScoreOptions{softcap, sink, chunk, rel, n_dist});
 }
 
 // Can the causal kernel take the queries from the fused projection itself (norm, rotation over `rot` features)?
@@ -1309,10 +1342,12 @@ DRYFT_API int dryft_attn_split_bf16(const void* q, const void* k_pages, const vo
                                     int max_pages, const int* seq_slot, const int* cu_rows, const int* kv_len,
                                     int n_seqs, float* part_o, float* part_ml, int n_splits, void* out, int n_heads,
                                     int n_kv, int head_dim, float scale, int window, float softcap, const float* sink,
-                                    hipStream_t stream) {
+                                    int chunk, const float* rel, int n_dist, hipStream_t stream) {
   FusedQKV none = {};
+  if (chunk < 0 || (chunk > 0 && window > 0) || (rel != nullptr && n_dist <= 0)) return -1;
   return launch_split(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, kv_len, n_seqs, part_o, part_ml,
-                      n_splits, out, n_heads, n_kv, head_dim, scale, window, none, stream, ScoreOptions{softcap, sink});
+                      n_splits, out, n_heads, n_kv, head_dim, scale, window, none, stream,
+                      ScoreOptions{softcap, sink, chunk, rel, n_dist});
 }
 
 // The same with the work of the norm/rotation/append kernel folded in: `qkv` is the fused projection's output

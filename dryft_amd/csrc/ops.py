@@ -55,12 +55,12 @@ _SIGNATURES = {
                                               _I, _I, _I, _P]},
     "attn_rows": {"dryft_attn_rows": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P, _I, _I, _P, _I, _I, _P]},
     "attn_mfma": {"dryft_attn_causal_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _F, _I, _I, _F, _P,
-                                             _P],
+                                             _I, _P, _I, _P],
                   "dryft_attn_causal_takes_projection": [_I, _I],
                   "dryft_attn_causal_projected_bf16": [_P, _L, _P, _I, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I,
                                                        _I, _P, _I, _I, _I, _F, _I, _I, _P],
                   "dryft_attn_split_bf16": [_P, _P, _P, _P, _I, _P, _P, _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I,
-                                            _F, _P, _P],
+                                            _F, _P, _I, _P, _I, _P],
                   "dryft_attn_decode_fused_bf16": [_P, _L, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _I, _P, _P, _P, _I, _P, _P,
                                                    _P, _I, _P, _P, _I, _P, _I, _I, _I, _F, _I, _P]},
     "gemm": {"dryft_gemm_tiled": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
@@ -578,12 +578,15 @@ ATTN_ROW_TILE = 64      # rows of a sequence that one workgroup of the prompt-at
 
 def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu, seq_start, n_seqs: int,
                      max_tiles: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int,
-                     mode: int = 0, softcap: float = 0.0, sink=None) -> None:
+                     mode: int = 0, softcap: float = 0.0, sink=None, chunk: int = 0, rel=None) -> None:
     """Causal attention of steps with many rows per sequence. ``mode``: 0 lets the library choose how much a wave
     takes; 1 = one head and 16 rows, 2 = two heads of a kv group, 3 = one head and 32 rows. At head size 128, 1 and
     3 bring the pages straight into LDS; 5 and 7 are 1 and 3 with the pages staged through registers, as at every
-    other head size. ``softcap`` > 0 caps the scores, ``sink`` (float32 ``[heads]``) joins each head's denominator."""
+    other head size. ``softcap`` > 0 caps the scores, ``sink`` (float32 ``[heads]``) joins each head's denominator;
+    ``chunk`` > 0: a row sees the earlier keys of its own run of so many positions (no window then); ``rel``: float32
+    ``[distances, heads]``, a bias by distance added to the scaled score (the last row for every larger distance)."""
     _check_sink(sink, n_heads)
+    _check_rel(rel, n_heads)
     _gpu(q, "q", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     if not (q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel()):
@@ -599,7 +602,8 @@ def attn_causal_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, tile_cu
     _check(_fn("attn_mfma", "dryft_attn_causal_bf16")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(tile_cu), _ptr(seq_start), n_seqs, max_tiles, _ptr(out), n_heads, n_kv, head_dim, float(scale),
-        int(window), int(mode), float(softcap), _ptr(sink), _stream()), "attn_causal_bf16")
+        int(window), int(mode), float(softcap), _ptr(sink), int(chunk), _ptr(rel),
+        rel.shape[0] if rel is not None else 0, _stream()), "attn_causal_bf16")
 
 
 def attn_causal_takes_projection(head_dim: int, rot: int) -> bool:
@@ -651,8 +655,9 @@ def attn_causal_projected_bf16(qkv, q_weight, eps: float, cos, sin, k_pages, v_p
 
 def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, n_seqs: int, part_o, part_ml,
                     n_splits: int, out, n_heads: int, n_kv: int, head_dim: int, scale: float, window: int,
-                    softcap: float = 0.0, sink=None) -> None:
+                    softcap: float = 0.0, sink=None, chunk: int = 0, rel=None) -> None:
     _check_sink(sink, n_heads)
+    _check_rel(rel, n_heads)
     _gpu(q, "q", torch.bfloat16)
     _gpu(out, "out", torch.bfloat16)
     if not (q.is_contiguous() and out.is_contiguous() and out.numel() == q.numel()):
@@ -672,7 +677,8 @@ def attn_split_bf16(q, k_pages, v_pages, page_table, seq_slot, cu_rows, kv_len, 
     _check(_fn("attn_mfma", "dryft_attn_split_bf16")(
         _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(page_table), page_table.shape[1], _ptr(seq_slot), _ptr(cu_rows),
         _ptr(kv_len), n_seqs, _ptr(part_o), _ptr(part_ml), n_splits, _ptr(out), n_heads, n_kv, head_dim, float(scale),
-        int(window), float(softcap), _ptr(sink), _stream()), "attn_split_bf16")
+        int(window), float(softcap), _ptr(sink), int(chunk), _ptr(rel), rel.shape[0] if rel is not None else 0,
+        _stream()), "attn_split_bf16")
 
 
 def attn_decode_fused_bf16(qkv, q_weight, k_weight, eps: float, cos, sin, rot: int, write_kv: bool, k_pages, v_pages,

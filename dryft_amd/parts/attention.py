@@ -234,8 +234,7 @@ class GQAAttention(Mixer):
                                   line.page_table, writes_cache, H, G, D, Dv)
         # bfloat16 on the matrix cores where they take the sizes (keys and values of one width, a multiple of 16);
         # float32, and the other sizes, on the kernel that takes one (row, head) a workgroup in float arithmetic
-        matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0 and \
-            not self.chunk and self.rel is None
+        matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0
         window = self.window or 0
         if matrix_cores and ctx.max_q_len == 1:
             out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
@@ -244,7 +243,7 @@ class GQAAttention(Mixer):
             part_ml = torch.empty((ctx.n_seqs, H, splits, 2), dtype=torch.float32, device=h.device)
             ops.attn_split_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, ctx.kv_len, ctx.n_seqs,
                                 part_o, part_ml, splits, out, H, G, D, self.scale, window, softcap=self.softcap,
-                                sink=self.sink)
+                                sink=self.sink, chunk=self.chunk or 0, rel=self.rel)
         elif matrix_cores:
             # the tiled kernel never visits the rows of sequences that sit out; they must hold something finite
             out = ctx.kept_zeros((rows, H, Dv), h.dtype) if ctx.some_sit_out() else \
@@ -252,7 +251,7 @@ class GQAAttention(Mixer):
             tile_cu, max_tiles = ctx.tiles(ops.ATTN_ROW_TILE)
             ops.attn_causal_bf16(q, line.k, line.v, line.page_table, ctx.seq_slot, ctx.cu_rows, tile_cu, ctx.seq_start,
                                  ctx.n_seqs, max_tiles, out, H, G, D, self.scale, window, softcap=self.softcap,
-                                 sink=self.sink)
+                                 sink=self.sink, chunk=self.chunk or 0, rel=self.rel)
         else:
             out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, G, D, self.scale,
