@@ -134,7 +134,8 @@ def compare_fetedra(args, design: str = "fetedra", relative: str = "piralix") ->
     the presets of a width hold about the same weight bytes); random weights, bfloat16, one prompt of
     ``--prompt-len`` tokens and ``--batch`` sequences decoding. One JSON line. ``--design barilix`` does the same for
     Barilix beside the Fetedra preset of the same width (recurrent and windowed-attention layers with experts on a
-    float32 stream, as many layers of the same widths)."""
+    float32 stream, as many layers of the same widths), ``--design podenex`` for Podenex beside it (three kinds of
+    windowed or chunked attention, one of them Fetedra's latent kind, with routed experts on a float32 stream)."""
     import torch
 
     from dryft_amd import Engine
@@ -162,9 +163,9 @@ def compare_fetedra(args, design: str = "fetedra", relative: str = "piralix") ->
 def main() -> int:
     global PROMPT, SLOT
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["piralix", "fetedra", "barilix"],
+    ap.add_argument("--design", default=None, choices=["piralix", "fetedra", "barilix", "podenex"],
                     help="instead of the default workload: that design beside its closest relative in the library at "
-                         "equal size (Piralix beside Qwen3, Fetedra beside Piralix, Barilix beside Fetedra; one JSON line)")
+                         "equal size (Piralix beside Qwen3, Fetedra beside Piralix, Barilix and Podenex beside Fetedra; one JSON line)")
     ap.add_argument("--sizes", default=None, help="presets for --design (default: the design's presets)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
@@ -188,9 +189,10 @@ def main() -> int:
     if args.design:
         args.sizes = args.sizes or {"piralix": "piralix-w1024,piralix-w2048,piralix-w2560",
                                     "fetedra": "fetedra-w1024,fetedra-w2048",
-                                    "barilix": "barilix-w1024,barilix-w2048"}[args.design]
-        if args.design == "barilix":
-            return compare_fetedra(args, "barilix", "fetedra")
+                                    "barilix": "barilix-w1024,barilix-w2048",
+                                    "podenex": "podenex-w1024,podenex-w2048"}[args.design]
+        if args.design in ("barilix", "podenex"):
+            return compare_fetedra(args, args.design, "fetedra")
         return compare_fetedra(args) if args.design == "fetedra" else compare_designs(args)
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (asked for {args.gpus}); this library has no multi-GPU path")

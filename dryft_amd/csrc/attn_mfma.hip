@@ -386,16 +386,34 @@ __device__ __forceinline__ void locate_tile(int tile, const int* __restrict__ se
 // A wave serves U = GP * RP units: GP query heads of one kv group, each over RP tiles of 16 consecutive rows. Every
 // piece of a page that a wave reads from LDS is used for all its units, so two units halve the LDS reads per
 // matrix instruction. A workgroup's tile is 64 * RP rows.
+// bytes of LDS the pages of the kernel below take: two pages of keys [64][D+8] and two of values [D][64+8] (one with
+// one unit per wave)
+__host__ __device__ constexpr size_t causal_page_bytes(int head_dim, int units) {
+  return (2 * (size_t)PAGE_TOKENS * (head_dim + 8) + (units == 1 ? 1 : 2) * (size_t)head_dim * (PAGE_TOKENS + 8)) * 2;
+}
+#define CAUSAL_REL_LDS_BYTES (16 * 1024)     // the most a bias table may take there
+
 template <int KB, bool FULL, int GP, int RP>
 __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1 ? 3 : 2) : 1) void attn_causal_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window, ScoreOptions opt) {
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int head_dim, float scale, int window, ScoreOptions opt,
+    int rel_lds) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   constexpr int U = GP * RP, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP;
-  const ScoreCap cap = score_cap(opt, scale, n_heads);
+  ScoreCap cap = score_cap(opt, scale, n_heads);
   const int chunk = opt.chunk;
+  // A small bias table waits in LDS behind the pages, one column per head of the wave: a score's look-up is then
+  // an LDS read of neighbouring words instead of a trip to the vector cache (`rel_lds`: the host says so).
+  float* const rel_held = (float*)(lds_raw + causal_page_bytes(head_dim, U));
+  if (rel_lds) {
+    const int head_base = (GP != 1 ? blockIdx.y : blockIdx.x) * GP;
+    for (int i = threadIdx.x; i < GP * opt.n_dist; i += blockDim.x)
+      rel_held[i] = opt.rel[(int64_t)(i % opt.n_dist) * n_heads + head_base + i / opt.n_dist];
+    cap.rel = rel_held;                                       // read only behind the first barrier of the walk
+    cap.rel_stride = 1;
+  }
   // Two heads per wave: a workgroup takes one tile from each end of the list (grid: pairs of tiles x heads / 2).
   // Otherwise: one tile per workgroup, the ones with the most pages first, heads fastest (grid: heads x tiles),
   // so that the short tiles fill the compute units that the long ones leave.
@@ -502,7 +520,7 @@ __global__ __launch_bounds__(256, (GP * RP * KB <= 8 && KB <= 4) ? (GP * RP == 1
         // or a chunk's start
         const bool masked = key0 + PAGE_TOKENS - 1 > pos0[rt] || rows[rt] < 16 ||
                             key0 < first_seen(pos0[rt] + 15, window, chunk);
-        const ScoreCap mine = for_head(cap, head0 + u % GP);
+        const ScoreCap mine = for_head(cap, rel_lds ? (u % GP) * opt.n_dist : head0 + u % GP);
         alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], mine)
                           : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[rt], pos_row[rt], moved[u], mine);
       }
@@ -673,12 +691,15 @@ __device__ __forceinline__ void init_rows_projected(RowBlock<4>& st, const Proje
 // latency than a second buffer would (0.67 against 0.63 PFLOP/s at 3,000 positions, 0.76 against 0.70 at 4,096,
 // the same at 2,048). With 32 rows a wave the registers allow two workgroups a unit anyway, so both have two
 // buffers and a page takes one barrier.
-template <int RP>
+// EXTRA: the form that also knows chunks and a sink (a build of its own, so that the plain form keeps its registers).
+template <int RP, bool EXTRA>
 __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     const int* __restrict__ page_table, int max_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_rows, const int* __restrict__ tile_cu, const int* __restrict__ seq_start, int n_seqs,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, float scale, int window, ProjectedQ projected) {
+    bf16_t* __restrict__ out, int n_heads, int n_kv, float scale, int window, ProjectedQ projected, int chunk_given,
+    const float* __restrict__ sink, const float* __restrict__ rel, int n_dist) {
+  const int chunk = EXTRA ? chunk_given : 0;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   constexpr int KB = DIRECT_D / 32, TILE_ROWS = 64 * RP, WAVE_ROWS = 16 * RP, head_dim = DIRECT_D;
   constexpr bool TWO = RP != 1;                               // two buffers each for keys and values
@@ -709,18 +730,29 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
     row[rt] = (int64_t)cu_rows[seq] + first + c;
     pos0[rt] = pos_wave + 16 * rt;
     pos_row[rt] = row_valid[rt] ? pos0[rt] + c : -1;
-    lo_row[rt] = window > 0 ? max(0, pos_row[rt] - window + 1) : 0;
+    lo_row[rt] = first_seen(pos_row[rt], window, chunk);
     if (projected.qkv != nullptr)
       init_rows_projected(st[rt], projected, row[rt], head, pos0[rt] + c, row_valid[rt]);
     else
       init_rows<KB>(st[rt], q + (row[rt] * n_heads + head) * head_dim, row_valid[rt], head_dim);
   }
   const int kvh = head / (n_heads / n_kv);
-  const int lo_wave = window > 0 ? max(0, pos_wave - window + 1) : 0;
+  const int lo_wave = first_seen(pos_wave, window, chunk);
   const int hi_wave = pos_wave + wave_rows - 1;
-  const int lo_tile = window > 0 ? max(0, pos_tile - window + 1) : 0;
+  const int lo_tile = first_seen(pos_tile, window, chunk);
   const int hi_tile = pos_tile + min(TILE_ROWS, q_len - tile_first) - 1;
-  const float scale_log2 = scale * 1.44269504088896340736f;
+  // EXTRA, a bias by distance: the head's column of the table waits in LDS behind the pages (the host has made
+  // room); it is read only behind the first barrier of the walk
+  ScoreCap cap;
+  if (EXTRA && rel != nullptr) {
+    float* held = (float*)(lds_raw + (RP == 1 ? 2 : 4) * DIRECT_PAGE_BYTES);
+    for (int i = threadIdx.x; i < n_dist; i += blockDim.x) held[i] = rel[(int64_t)i * n_heads + head];
+    cap.rel = held;
+    cap.rel_stride = 1;
+    cap.n_dist = n_dist;
+    cap.rel_scale = scale;
+  }
+  const float scale_log2 = (EXTRA && rel != nullptr ? 1.f : scale) * 1.44269504088896340736f;
   const int64_t page_elems = (int64_t)PAGE_TOKENS * head_dim;
   const int* table = page_table + (int64_t)slot * max_pages;
   const int pg_first = lo_tile / PAGE_TOKENS, pg_last = hi_tile / PAGE_TOKENS;
@@ -773,9 +805,9 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
 #pragma unroll
       for (int u = 0; u < RP; ++u) {
         const bool masked = key0 + PAGE_TOKENS - 1 > pos0[u] || rows[u] < 16 ||
-                            (window > 0 && key0 < pos0[u] + 15 - window + 1);
-        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[u], pos_row[u], moved[u])
-                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[u], pos_row[u], moved[u]);
+                            key0 < first_seen(pos0[u] + 15, window, chunk);
+        alpha[u] = masked ? page_softmax<KB, true>(st[u], s[u], p[u], scale_log2, key0, lo_row[u], pos_row[u], moved[u], EXTRA ? cap : ScoreCap{})
+                          : page_softmax<KB, false>(st[u], s[u], p[u], scale_log2, key0, lo_row[u], pos_row[u], moved[u], EXTRA ? cap : ScoreCap{});
       }
 #pragma unroll
       for (int u = 0; u < RP; ++u)
@@ -806,6 +838,7 @@ __global__ __launch_bounds__(256, RP == 1 ? 4 : 2) void attn_causal_direct_kerne
 #pragma unroll
   for (int u = 0; u < RP; ++u) {
     if (!row_valid[u]) continue;
+    if (EXTRA && sink != nullptr) row_l[u] += sink_term(sink, head, st[u].m);
     const float inv = 1.f / row_l[u];
     bf16_t* o = out + (row[u] * n_heads + head) * head_dim;
 #pragma unroll
@@ -1191,7 +1224,9 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
   if (GP == 1) grid = dim3(n_heads, RP == 1 ? max_tiles : (max_tiles + n_seqs + 1) / 2);
   if (grid.y > 65535) return -1;
   // two pages of keys [64][D+8] and two of values [D][64+8] (one with one unit per wave)
-  const size_t lds = (2 * (size_t)PAGE_TOKENS * (head_dim + K_PAD) + (GP * RP == 1 ? 1 : 2) * (size_t)head_dim * (PAGE_TOKENS + V_PAD)) * 2;
+  const size_t rel_bytes = opt.rel != nullptr ? (size_t)GP * opt.n_dist * sizeof(float) : 0;
+  const int rel_lds = rel_bytes > 0 && rel_bytes <= CAUSAL_REL_LDS_BYTES;
+  const size_t lds = causal_page_bytes(head_dim, GP * RP) + (rel_lds ? rel_bytes : 0);
 #define LAUNCH_CAUSAL(FULLV)                                                                                       \
   {                                                                                                                \
     auto kernel = attn_causal_kernel<KB, FULLV, GP, RP>;                                                           \
@@ -1200,7 +1235,7 @@ static int launch_causal(const void* q, const void* k_pages, const void* v_pages
       return -1;                                                                                                   \
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, (const bf16_t*)q, (const bf16_t*)k_pages,                 \
                        (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs, \
-                       (bf16_t*)out, n_heads, n_kv, head_dim, scale, window, opt);                                 \
+                       (bf16_t*)out, n_heads, n_kv, head_dim, scale, window, opt, rel_lds);                        \
   }
   if (head_dim % 32 == 0) {
     DISPATCH_KB(head_dim / 32, LAUNCH_CAUSAL(true));
@@ -1215,14 +1250,23 @@ template <int RP>
 static int launch_causal_direct(const void* q, const void* k_pages, const void* v_pages, const int* page_table,
                                 int max_pages, const int* seq_slot, const int* cu_rows, const int* tile_cu,
                                 const int* seq_start, int n_seqs, int max_tiles, void* out, int n_heads, int n_kv,
-                                float scale, int window, ProjectedQ projected, hipStream_t stream) {
+                                float scale, int window, ProjectedQ projected, hipStream_t stream, int chunk = 0,
+                                const float* sink = nullptr, const float* rel = nullptr, int n_dist = 0) {
   // max_tiles bounds the 64-row tiles of the sequences that take part; a sequence with t of them has ceil(t / RP)
   dim3 grid(n_heads, (max_tiles + (RP - 1) * (n_seqs + 1)) / RP), block(256);
   if (grid.y > 65535) return -1;
-  const size_t lds = (size_t)(RP == 1 ? 2 : 4) * DIRECT_PAGE_BYTES;
-  hipLaunchKernelGGL(attn_causal_direct_kernel<RP>, grid, block, lds, stream, (const bf16_t*)q, (const bf16_t*)k_pages,
-                     (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start, n_seqs,
-                     (bf16_t*)out, n_heads, n_kv, scale, window, projected);
+  const size_t lds = (size_t)(RP == 1 ? 2 : 4) * DIRECT_PAGE_BYTES + (rel != nullptr ? (size_t)n_dist * sizeof(float) : 0);
+  if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)attn_causal_direct_kernel<RP, true>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return -1;
+  if (chunk > 0 || sink != nullptr || rel != nullptr)
+    hipLaunchKernelGGL((attn_causal_direct_kernel<RP, true>), grid, block, lds, stream, (const bf16_t*)q,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu,
+                       seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, scale, window, projected, chunk, sink, rel, n_dist);
+  else
+    hipLaunchKernelGGL((attn_causal_direct_kernel<RP, false>), grid, block, lds, stream, (const bf16_t*)q,
+                       (const bf16_t*)k_pages, (const bf16_t*)v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu,
+                       seq_start, n_seqs, (bf16_t*)out, n_heads, n_kv, scale, window, projected, 0, nullptr, nullptr, 0);
   return DRYFT_LAUNCH_CHECK();
 }
 
@@ -1239,9 +1283,10 @@ static int causal_entry(const void* q, const void* k_pages, const void* v_pages,
   const bool staged = mode == 5 || mode == 7;
   if (staged) mode -= 4;
   if (mode < 0 || mode > 3 || (mode == 2 && (group % 2 || head_dim > 128)) || (mode == 3 && head_dim > 128)) return -1;
-  // (the kernel that brings pages straight into LDS knows neither a cap nor a sink, chunks or a bias)
+  // (the kernel that brings pages straight into LDS knows no cap, and a bias by distance only where its table fits LDS)
   const bool direct_ok = head_dim == DIRECT_D && (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0 &&
-                         !(opt.softcap > 0.f) && opt.sink == nullptr && opt.chunk == 0 && opt.rel == nullptr;
+                         !(opt.softcap > 0.f) &&
+                         (opt.rel == nullptr || (size_t)opt.n_dist * sizeof(float) <= CAUSAL_REL_LDS_BYTES);
   if (mode == 0) {
     // Two units per wave (twice the rows of one head, or two heads of a kv group) use every piece of a page that
     // is read from LDS twice; they also halve the number of workgroups, so they need four of them for every
@@ -1262,9 +1307,11 @@ static int causal_entry(const void* q, const void* k_pages, const void* v_pages,
   if (direct_ok && !staged && mode != 2) {
     if (mode == 3)
       return launch_causal_direct<2>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
-                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, projected, stream);
+                                     n_seqs, max_tiles, out, n_heads, n_kv, scale, window, projected, stream, opt.chunk,
+                                     opt.sink, opt.rel, opt.n_dist);
     return launch_causal_direct<1>(q, k_pages, v_pages, page_table, max_pages, seq_slot, cu_rows, tile_cu, seq_start,
-                                   n_seqs, max_tiles, out, n_heads, n_kv, scale, window, projected, stream);
+                                   n_seqs, max_tiles, out, n_heads, n_kv, scale, window, projected, stream, opt.chunk,
+                                   opt.sink, opt.rel, opt.n_dist);
   }
   if (projected.qkv != nullptr) return -1;                   // only the kernel above takes the projection itself
   if (mode == 2) CAUSAL(2, 1);

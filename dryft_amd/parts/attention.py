@@ -157,7 +157,9 @@ class GQAAttention(Mixer):
             rows, far = tensors["rel"].shape[0], self.distance_bias[1]
             if not 2 <= rows < 2 * far:
                 raise ValueError(f"a bias table of {rows} rows does not go with a far distance of {far}")
-            index = torch.tensor([distance_row(n, rows, far) for n in range(far + 1)], device=self.w_qkv.device)
+            reach = self.chunk or self.window                      # no row looks further back than that
+            last = min(far, reach - 1) if reach else far
+            index = torch.tensor([distance_row(n, rows, far) for n in range(last + 1)], device=self.w_qkv.device)
             self.rel = tensors["rel"].float()[index].contiguous()
         if self.value_mix:
             self.vmix = tensors["vmix"].float().reshape(1).contiguous()

@@ -180,6 +180,8 @@ MIXER_SHAPES = {
     "chunked-bare": chunked(3, 3, 20, 12, conv=1),                         # one tap, no chunk, no table
     "chunked-no-conv": chunked(2, 2, 64, 64, chunk=100, bias=(32, 64)),
     "chunked-128": chunked(2, 1, 128, 128, conv=4, chunk=128, bias=(16, 120), scale=0.05),
+    "chunked-128-no-table": chunked(2, 1, 128, 128, conv=2, chunk=100, scale=0.05),
+    "chunked-long-table": chunked(2, 2, 32, 32, bias=(8, 5000)),          # too long for LDS: read from memory
     "sinked-cores": sinked(4, 2, 32, 32, window=20, v_mix=True),
     "sinked-wide-values": sinked(2, 1, 24, 64, window=65),
     "sinked-odd": sinked(6, 3, 10, 12),
