@@ -134,6 +134,64 @@ def test_token_side_part(dtype):
     assert rel_err(got, want) <= MIXER_TOL[dtype]
 
 
+@pytest.mark.parametrize("options", ["chunk", "chunk+bias", "window+sink", "bias+sink", "chunk+bias+sink"])
+@pytest.mark.parametrize("heads,kv,D,lengths,tq", [(8, 2, 128, [700, 330, 65], 290), (4, 2, 32, [300, 129, 70], 300),
+                                                    (6, 2, 64, [200, 150, 1], 1), (16, 4, 128, [2100], 2100)])
+def test_attention_options_on_the_matrix_cores(options, heads, kv, D, lengths, tq):
+    """Chunks, the bias by distance and a sink in every way of running the prompt kernel (16 or 32 rows a wave, two
+    heads a wave, pages staged or straight into LDS, a bias table in LDS or too long for it) and in the decode kernel,
+    against dense float64 arithmetic; rows continue after cached tokens, and chunks are counted from position 0."""
+    from dryft_amd.csrc import ops
+    from helpers import build_pages
+    g = torch.Generator().manual_seed(len(options) + D)
+    B, L = len(lengths), max(lengths)
+    chunk = 100 if "chunk" in options else 0
+    window = 90 if "window" in options else 0
+    sink = torch.full((heads,), 0.0) if "sink" in options else None
+    scale = 1.5 / D ** 0.5
+    k = torch.randn(B, L, kv, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, L, kv, D, generator=g).to(torch.bfloat16)
+    q_lens = [min(tq, n) for n in lengths]
+    q = torch.randn(B, max(q_lens), heads, D, generator=g).to(torch.bfloat16)
+    k_pages, v_pages, table, slots = build_pages(k, v, lengths, sum((n + 63) // 64 for n in lengths) + 3, B + 2, seed=1, poison=1e4)
+    cu = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    tiles = np.concatenate([[0], np.cumsum([(ql + 63) // 64 for ql in q_lens])]).astype(np.int32)
+    q_packed = torch.cat([q[b, :ql] for b, ql in enumerate(q_lens)]).contiguous()
+    d = lambda t: t.to(DEV)                                                    # noqa: E731
+    for n_dist in ((40, 5000) if "bias" in options else (0,)):
+        rel = 2 * torch.randn(n_dist, heads, generator=g) if n_dist else None
+        want = []
+        for b, (n, ql) in enumerate(zip(lengths, q_lens)):
+            pos_q, pos_k = torch.arange(n - ql, n), torch.arange(n)
+            sc = torch.einsum("qhd,khd->hqk", q[b, :ql].double(), k[b, :n].double().repeat_interleave(heads // kv, 1)) * scale
+            if rel is not None:
+                sc = sc + rel.double()[(pos_q[:, None] - pos_k[None, :]).clamp(0, n_dist - 1)].permute(2, 0, 1)
+            mask = P.chunk_mask(pos_q, pos_k, chunk) if chunk else P.window_mask(pos_q, pos_k, window or None)
+            want.append(P.weigh(sc, mask, v[b, :n].double(), heads // kv, sink=sink is not None))
+        want = torch.cat(want)
+        common = dict(sink=d(sink) if sink is not None else None, chunk=chunk, rel=d(rel) if rel is not None else None)
+        seq_slot = d(torch.tensor(slots, dtype=torch.int32))
+        if tq == 1:
+            for splits in (1, 3):
+                out = torch.zeros(sum(q_lens), heads, D, dtype=torch.bfloat16, device=DEV)
+                part_o = torch.empty(B * heads * splits * D, dtype=torch.float32, device=DEV)
+                part_ml = torch.empty(B * heads * splits * 2, dtype=torch.float32, device=DEV)
+                ops.attn_split_bf16(d(q_packed), d(k_pages), d(v_pages), d(table), seq_slot, d(torch.from_numpy(cu)),
+                                    d(torch.tensor(lengths, dtype=torch.int32)), B, part_o, part_ml, splits, out, heads, kv, D,
+                                    scale, window, **common)
+                assert rel_err(out, want) <= 2e-2, (options, n_dist, splits)
+            continue
+        for mode in (0, 1, 2, 3, 5, 7):
+            if mode in (2, 3, 7) and D > 128:
+                continue
+            out = torch.zeros(sum(q_lens), heads, D, dtype=torch.bfloat16, device=DEV)
+            ops.attn_causal_bf16(d(q_packed), d(k_pages), d(v_pages), d(table), seq_slot, d(torch.from_numpy(cu)),
+                                 d(torch.from_numpy(tiles)),
+                                 d(torch.tensor([n - ql for n, ql in zip(lengths, q_lens)], dtype=torch.int32)), B,
+                                 int(tiles[-1]) + 1, out, heads, kv, D, scale, window, mode, **common)
+            assert rel_err(out, want) <= 2e-2, (options, n_dist, mode)
+
+
 # ------------------------------------------------------------------------------------------ mixers alone
 def mixer_case(layer, width, seed):
     from dryft_amd.config.podenex import PodenexConfig
