@@ -49,7 +49,7 @@ _SIGNATURES = {
                 "dryft_rope_pairs_kv": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                         _I, _I, _P],
                 "dryft_norm_rope_half_kv": [_P, _L, _I, _I, _I, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I,
-                                            _I, _I, _I, _I, _I, _P],
+                                            _I, _I, _I, _I, _I, _I, _P],
                 "dryft_rows_to_cache_takes": [_I, _I, _I, _I],
                 "dryft_rows_to_cache_parts": [_P, _I, _L, _P, _P, _I, _I, _F, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I,
                                               _I, _I, _I, _P]},
@@ -1899,11 +1899,13 @@ def conv_tail(u, col: int, channels: int, in_bias, taps: int, seq_slot, cu_rows,
 # ------------------------------------------------------------------------- norm per head, rotation over halves, append
 def norm_rope_half_kv(src, q_col: int, k_col: int, v_col: int, q_weight, k_weight, eps: float, cos, sin, rot: int,
                       row_slot, row_pos, q_out, k_pages, v_pages, page_table, write_kv: bool, n_heads: int, n_kv: int,
-                      head_dim: int, v_dim: int) -> None:
+                      head_dim: int, v_dim: int, page_dim: int = 0) -> None:
     """Every q and k head of ``src`` divided by its root mean square and multiplied by ``q_weight`` / ``k_weight``
     (float32 ``[head_dim]``; None: the head passes), then feature ``i`` of its first ``rot`` turned with feature
     ``i + rot / 2`` by float32 tables ``[positions, rot / 2]``; queries to ``q_out [rows, heads, head_dim]`` and, when
-    ``write_kv``, keys and (untouched) values of width ``v_dim`` to their pages."""
+    ``write_kv``, keys and (untouched) values of width ``v_dim`` to their pages. ``page_dim`` > 0: pages and the rows of
+    ``q_out`` are that wide for keys and values alike (at least as wide as either); what lies behind a head's own
+    features is not written, so ``q_out`` and the pages must have started as zeros."""
     _gpu(src, "src")
     is_f32 = _float_flag(src, "src")
     rows = src.shape[0]
@@ -1923,14 +1925,17 @@ def norm_rope_half_kv(src, q_col: int, k_col: int, v_col: int, q_weight, k_weigh
         if t is not None:
             _f32_vector(t, name, head_dim)
     _gpu(q_out, "q_out", src.dtype)
-    if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * head_dim):
+    page_dim = int(page_dim)
+    if page_dim and page_dim < max(head_dim, v_dim):
+        raise KernelError("norm_rope_half_kv: padded pages must be at least as wide as keys and values")
+    if not (q_out.is_contiguous() and q_out.numel() == rows * n_heads * (page_dim or head_dim)):
         raise KernelError("norm_rope_half_kv: q_out must be [rows, heads, head_dim]")
-    _check_pages(k_pages, v_pages, page_table, n_kv, head_dim, src.dtype, v_dim)
+    _check_pages(k_pages, v_pages, page_table, n_kv, page_dim or head_dim, src.dtype, page_dim or v_dim)
     _row_facts(rows, row_slot=row_slot, row_pos=row_pos)
     _check(_fn("rope_kv", "dryft_norm_rope_half_kv")(
         _ptr(src), src.stride(0), q_col, k_col, v_col, _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(cos), _ptr(sin),
         rot, _ptr(row_slot), _ptr(row_pos), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(page_table),
-        page_table.shape[1], int(bool(write_kv)), rows, n_heads, n_kv, head_dim, v_dim, is_f32, _stream()),
+        page_table.shape[1], int(bool(write_kv)), rows, n_heads, n_kv, head_dim, v_dim, page_dim, is_f32, _stream()),
         "norm_rope_half_kv")
 
 

@@ -660,6 +660,9 @@ DRYFT_API int dryft_rope_pairs_kv(const void* proj, int64_t proj_stride, int q_c
 //
 // and features from `rot` on pass. All of it is float arithmetic, rounded once on the way out. The row's q, k and v
 // start at columns q_col, k_col and v_col of `src`. One wave per head; the head waits in LDS between norm and turn.
+// With `page_dim` > 0 the pages (and the rows of q_out) are that wide for keys and values alike, wider than either:
+// a head's features go to the front of its row, and what lies behind them is never written (it holds the zeros it
+// started with), so that kernels which take one width for keys and values serve heads whose widths differ.
 #define NRH_MAX_DIM 256
 
 template <typename T>
@@ -668,8 +671,9 @@ __global__ __launch_bounds__(256) void norm_rope_half_kv_kernel(
     const float* __restrict__ k_w, float eps, const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot,
     const int* __restrict__ row_slot, const int* __restrict__ row_pos, T* __restrict__ q_out, T* __restrict__ k_pages,
     T* __restrict__ v_pages, const int* __restrict__ page_table, int max_pages, int write_kv, int n_heads, int n_kv,
-    int head_dim, int v_dim, int skip_v) {
+    int head_dim, int v_dim, int skip_v, int page_dim) {
   __shared__ float held[4][NRH_MAX_DIM];
+  const int k_wide = page_dim > 0 ? page_dim : head_dim, v_wide = page_dim > 0 ? page_dim : v_dim;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int64_t row = blockIdx.x;
   const int job = blockIdx.y * 4 + wave;  // [0,nH): q heads; [nH,nH+nKV): k heads; then v heads
@@ -678,8 +682,8 @@ __global__ __launch_bounds__(256) void norm_rope_half_kv_kernel(
   const bool is_q = job < n_heads, is_k = !is_q && job < n_heads + n_kv;
   if (is_q) {
     if (slot < 0) {
-      T* dst = q_out + (row * n_heads + job) * head_dim;
-      for (int i = lane; i < head_dim; i += WAVE) store_from_float(dst + i, 0.f);
+      T* dst = q_out + (row * n_heads + job) * k_wide;
+      for (int i = lane; i < k_wide; i += WAVE) store_from_float(dst + i, 0.f);
       return;
     }
   } else if (slot < 0 || !write_kv) {
@@ -694,14 +698,14 @@ __global__ __launch_bounds__(256) void norm_rope_half_kv_kernel(
   if (!is_q && !is_k) {
     const int kvh = job - n_heads - n_kv;
     const T* src = src_rows + row * src_stride + v_col + (int64_t)kvh * v_dim;
-    T* dst = v_pages + ((int64_t)page * n_kv + kvh) * v_dim * PAGE_TOKENS + value_column(in_page);
+    T* dst = v_pages + ((int64_t)page * n_kv + kvh) * v_wide * PAGE_TOKENS + value_column(in_page);
     for (int i = lane; i < v_dim; i += WAVE) dst[(int64_t)i * PAGE_TOKENS] = src[i];
     return;
   }
   const T* src = src_rows + row * src_stride + (is_q ? q_col + (int64_t)job * head_dim
                                                      : k_col + (int64_t)(job - n_heads) * head_dim);
-  T* dst = is_q ? q_out + (row * n_heads + job) * head_dim
-                : k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + in_page) * head_dim;
+  T* dst = is_q ? q_out + (row * n_heads + job) * k_wide
+                : k_pages + (((int64_t)page * n_kv + (job - n_heads)) * PAGE_TOKENS + in_page) * k_wide;
   const float* w = is_q ? q_w : k_w;
   float* mine = held[wave];
   float ss = 0.f;
@@ -732,24 +736,25 @@ DRYFT_API int dryft_norm_rope_half_kv(const void* src, int64_t src_stride, int q
                                       const float* q_w, const float* k_w, float eps, const float* cos_t,
                                       const float* sin_t, int rot, const int* row_slot, const int* row_pos, void* q_out,
                                       void* k_pages, void* v_pages, const int* page_table, int max_pages, int write_kv,
-                                      int n_rows, int n_heads, int n_kv, int head_dim, int v_dim, int is_f32,
-                                      hipStream_t stream) {
+                                      int n_rows, int n_heads, int n_kv, int head_dim, int v_dim, int page_dim,
+                                      int is_f32, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (rot < 0 || rot % 2 || rot > head_dim || head_dim > NRH_MAX_DIM || n_kv <= 0 || q_out == nullptr) return -1;
+  if (page_dim != 0 && (page_dim < head_dim || page_dim < v_dim)) return -1;
   // many rows: the values are transposed a tile of 64 rows at a time instead of 2 bytes at a time
   const size_t v_lds = (size_t)v_dim * V_TILE_LD * (is_f32 ? 4 : 2);
-  const int skip_v = (write_kv && n_rows >= 32 && v_dim % 8 == 0 && v_col % 8 == 0 && src_stride % 8 == 0 &&
+  const int skip_v = (page_dim == 0 && write_kv && n_rows >= 32 && v_dim % 8 == 0 && v_col % 8 == 0 && src_stride % 8 == 0 &&
                       (((uintptr_t)src | (uintptr_t)v_pages) & 15) == 0 && v_lds <= 64 * 1024) ? 1 : 0;
   dim3 grid(n_rows, (n_heads + (skip_v ? 1 : 2) * n_kv + 3) / 4), block(256);
   if (is_f32)
     hipLaunchKernelGGL(norm_rope_half_kv_kernel<float>, grid, block, 0, stream, (const float*)src, src_stride, q_col,
                        k_col, v_col, q_w, k_w, eps, cos_t, sin_t, rot, row_slot, row_pos, (float*)q_out, (float*)k_pages,
-                       (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim, skip_v);
+                       (float*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim, v_dim, skip_v, page_dim);
   else
     hipLaunchKernelGGL(norm_rope_half_kv_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)src, src_stride, q_col,
                        k_col, v_col, q_w, k_w, eps, cos_t, sin_t, rot, row_slot, row_pos, (bf16_t*)q_out,
                        (bf16_t*)k_pages, (bf16_t*)v_pages, page_table, max_pages, write_kv, n_heads, n_kv, head_dim,
-                       v_dim, skip_v);
+                       v_dim, skip_v, page_dim);
   int rc = DRYFT_LAUNCH_CHECK();
   if (rc || !skip_v) return rc;
   dim3 vgrid((n_rows + V_TILE_ROWS - 1) / V_TILE_ROWS, n_kv);

@@ -39,7 +39,7 @@ def _norm(cfg: PodenexConfig, name: str) -> PartSpec:
 
 def _grouped(cfg: PodenexConfig, kind: str, m: dict, p: str, first_mix: bool) -> PartSpec:
     args = dict(hidden_size=cfg.width, num_heads=m["heads"], num_kv_heads=m["kv_heads"], head_dim=m["dim"],
-                value_dim=m["vdim"], scale=m["scale"], float_weights=True,
+                value_dim=m["vdim"], scale=m["scale"], float_weights=True, pad_pages=True,
                 value_mix=(VALUES, first_mix) if m["v_mix"] else None)
     names = {"q_proj": p + "q", "k_proj": p + "k", "v_proj": p + "v", "o_proj": p + "o"}
     if m["v_mix"]:

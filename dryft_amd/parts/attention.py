@@ -25,6 +25,11 @@ the first layer of that name leaves its values of the step's rows in the step co
 l) v + l v_first`` with its own learned ``l``, tensor ``vmix``, before anything is cached). Any of these takes the
 step down ``_forward_general``.
 
+``pad_pages``: in bfloat16, heads whose keys and values differ in width (or whose width is no multiple of 16) keep
+pages of one width for both, the next multiple of 16 that holds either, with zeros behind a head's own features: the
+matrix-core kernels, which take one width, then serve them (zeros add nothing to a score, and the outputs behind
+``value_dim`` are never read). Off by default; without it such heads take the float kernel.
+
 The part knows nothing of the model around it: sizes and constants are constructor arguments, the
 position encoding is looked up by name in the step context, and its storage is the cache line it
 is handed.
@@ -78,7 +83,8 @@ class GQAAttention(Mixer):
                  softcap: float | None = None, sink: bool = False, output_gate: bool | str = False,
                  float_weights: bool = False, bias: bool = False, conv_taps: int | None = None,
                  sink_value: float | None = None, chunk: int | None = None,
-                 distance_bias: tuple[int, int] | None = None, value_mix: tuple[str, bool] | None = None):
+                 distance_bias: tuple[int, int] | None = None, value_mix: tuple[str, bool] | None = None,
+                 pad_pages: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} kv heads evenly")
         if not 0 < head_dim <= MAX_HEAD_DIM:
@@ -110,6 +116,9 @@ class GQAAttention(Mixer):
             raise ValueError(f"a bias by distance needs at least 2 rows (-1: as many as the checkpoint holds) and a far "
                              f"distance beyond half of them, got {self.distance_bias}")
         self.value_mix = (str(value_mix[0]), bool(value_mix[1])) if value_mix else None
+        self.pad_pages = bool(pad_pages)
+        if self.pad_pages and positions:
+            raise ValueError("pages of one padded width go with mixers that do not rotate")
         self.q_dim, self.kv_dim = self.n_heads * self.head_dim, self.n_kv * self.head_dim
         self.v_dim, self.o_dim = self.n_kv * self.value_dim, self.n_heads * self.value_dim
         self.has_bias, self.conv_taps = bool(bias), int(conv_taps) if conv_taps else 0
@@ -121,7 +130,7 @@ class GQAAttention(Mixer):
                              self.chunk or self.distance_bias or self.value_mix)
         self.conv_channels = self.q_dim + self.kv_dim + self.v_dim
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.sink = None
-        self.in_bias = self.o_bias = self.conv_w = self.conv_wt = self.rel = self.vmix = None
+        self.in_bias = self.o_bias = self.conv_w = self.conv_wt = self.rel = self.vmix = self.w_o_padded = None
 
     def tensor_specs(self):
         specs = {"q_proj": matrix((self.q_dim, self.hidden)), "k_proj": matrix((self.kv_dim, self.hidden)),
@@ -164,6 +173,12 @@ class GQAAttention(Mixer):
         if self.value_mix:
             self.vmix = tensors["vmix"].float().reshape(1).contiguous()
         self.w_o = tensors["o_proj"]
+        wide = self.page_dim()
+        if wide and not self.output_gate:
+            # nothing packs the heads' outputs between attention and the projection: the projection skips the padding
+            padded = torch.zeros((self.hidden, self.n_heads, wide), dtype=self.w_o.dtype, device=self.w_o.device)
+            padded[:, :, :self.value_dim] = self.w_o.view(self.hidden, self.n_heads, self.value_dim)
+            self.w_o_padded = padded.view(self.hidden, self.n_heads * wide).contiguous()
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = tensors["q_norm"], tensors["k_norm"]
             if self.q_norm.dtype != self.k_norm.dtype or self.extended:   # one kernel argument says how both are stored
@@ -178,10 +193,20 @@ class GQAAttention(Mixer):
         if self.conv_w is not None:
             self.conv_wt = self.conv_w.t().contiguous()                  # tap by tap, for 8 channels a thread
 
+    def page_dim(self) -> int:
+        """The one width of keys' and values' pages where ``pad_pages`` applies (bfloat16, widths that differ or are
+        no multiple of the matrix cores' step, and the padded width within what the kernels take); else 0."""
+        D, Dv, step = self.head_dim, self.value_dim, MATRIX_CORE_HEAD_STEP
+        if not self.pad_pages or self.compute_dtype != torch.bfloat16 or (D == Dv and D % step == 0):
+            return 0
+        wide = -(-max(D, Dv) // step) * step
+        return wide if wide <= MAX_HEAD_DIM else 0
+
     def cache_need(self):
         # a row of a chunked mixer never looks further back than a chunk: the pages behind that are given back
-        kv = KVNeed(self.n_kv, self.head_dim, self.window or self.chunk,
-                    self.value_dim if self.value_dim != self.head_dim else None)
+        wide = self.page_dim()
+        kv = KVNeed(self.n_kv, wide or self.head_dim, self.window or self.chunk,
+                    self.value_dim if self.value_dim != self.head_dim and not wide else None)
         if self.conv_taps > 1:
             return {"kv": kv, "tail": conv_need(self.conv_taps, self.conv_channels)}
         return kv
@@ -224,7 +249,9 @@ class GQAAttention(Mixer):
                 if earlier is None or earlier.shape != v_cols.shape:
                     raise ValueError(f"values {name!r}: no earlier layer of this step has left values of this shape")
                 ops.blend_columns(v_cols, earlier, self.vmix)
-        q = torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
+        wide = self.page_dim()
+        q = torch.zeros((rows, H, wide), dtype=h.dtype, device=h.device) if wide else \
+            torch.empty((rows, H, D), dtype=h.dtype, device=h.device)
         if isinstance(table, PairRotaryPositions):
             if self.qk_norm_eps is not None:
                 raise NotImplementedError("per-head q/k norms do not go with the rotation over neighbouring pairs")
@@ -233,10 +260,12 @@ class GQAAttention(Mixer):
         else:
             ops.norm_rope_half_kv(src, 0, self.q_dim, self.q_dim + self.kv_dim, self.q_norm, self.k_norm,
                                   self.qk_norm_eps or 0.0, cos, sin, rot, ctx.row_slot, ctx.row_pos, q, line.k, line.v,
-                                  line.page_table, writes_cache, H, G, D, Dv)
-        # bfloat16 on the matrix cores where they take the sizes (keys and values of one width, a multiple of 16);
-        # float32, and the other sizes, on the kernel that takes one (row, head) a workgroup in float arithmetic
-        matrix_cores = h.dtype == torch.bfloat16 and D == Dv and D % MATRIX_CORE_HEAD_STEP == 0
+                                  line.page_table, writes_cache, H, G, D, Dv, page_dim=wide)
+        # bfloat16 on the matrix cores where they take the sizes (keys and values of one width, a multiple of 16, as
+        # they are or padded); float32, and the other sizes, on the kernel that takes one (row, head) a workgroup
+        matrix_cores = h.dtype == torch.bfloat16 and (wide or (D == Dv and D % MATRIX_CORE_HEAD_STEP == 0))
+        if wide:
+            D = Dv = wide                        # what the attention kernels see; o_dim keeps the values' own width
         window = self.window or 0
         if matrix_cores and ctx.max_q_len == 1:
             out = torch.empty((rows, H, Dv), dtype=h.dtype, device=h.device)
@@ -259,16 +288,18 @@ class GQAAttention(Mixer):
             ops.attn_rows(q, line.k, line.v, line.page_table, ctx.row_slot, ctx.row_pos, out, H, G, D, self.scale,
                           window, v_dim=Dv, softcap=self.softcap, sink=self.sink, exact_p=self.float_weights,
                           chunk=self.chunk or 0, rel=self.rel)
-        out = out.view(rows, self.o_dim)
         if self.output_gate:
-            gated = torch.empty_like(out)
+            gated = torch.empty((rows, self.o_dim), dtype=h.dtype, device=h.device)
             g_col = self.q_dim + self.kv_dim + self.v_dim
-            if self.head_gate:
-                ops.head_gate(out, proj, g_col, gated, H, Dv)
+            if self.head_gate or wide:           # this kernel also packs heads that are padded
+                ops.head_gate(out, proj, g_col, gated, H, self.value_dim, per_element=not self.head_gate)
                 out = gated
             else:
-                out = ops.sigmoid_gate(out, proj[:, g_col:g_col + self.o_dim], gated)
-        return linear(out, self.w_o, allow_partials=True)
+                out = ops.sigmoid_gate(out.view(rows, self.o_dim), proj[:, g_col:g_col + self.o_dim], gated)
+            return linear(out, self.w_o, allow_partials=True)
+        if wide:
+            return linear(out.view(rows, H * wide), self.w_o_padded, allow_partials=True)
+        return linear(out.view(rows, self.o_dim), self.w_o, allow_partials=True)
 
     def forward_split(self, h: torch.Tensor, ctx: StepContext, line, writes_cache: bool):
         if self.has_bias:
